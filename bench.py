@@ -1,0 +1,324 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE-forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_bf16|c4_fp8|c2_bf16|c5_bf16|c5_fp8]
+                    [--tokens T] [--no-cpu-baseline] [--no-extra]
+
+A step is one forward pass of the hot path over one batch of synthetic input that is
+already resident in HBM: top-k routing from the gate probabilities, the gather +
+grouped GEMM with its SiLU / SwiGLU epilogue, (fp8: the row-wise quantisations),
+the down-projection GEMM and the weighted merge.  The gate Linear + softmax that
+produce the probabilities stay torch calls and are outside the step, as they are
+outside the FLOP count.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK = {"bf16": 2500.0, "fp8": 5000.0}   # dense MFMA TFLOP/s, MI355X
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (T, E, K, D, H, O, kind, dtype, routing)
+    "c2_bf16": dict(T=8192, E=8, K=2, D=1024, H=4096, O=1024, kind="mlp", dtype="bf16", routing="gate"),
+    "c3_bf16": dict(T=16384, E=64, K=8, D=2048, H=1408, O=2048, kind="swiglu", dtype="bf16", routing="zipf"),
+    "c4_fp8": dict(T=16384, E=64, K=8, D=2048, H=1408, O=2048, kind="swiglu", dtype="fp8", routing="zipf"),
+    "c5_bf16": dict(T=4096, E=128, K=8, D=4096, H=1536, O=4096, kind="swiglu", dtype="bf16", routing="uniform"),
+    "c5_fp8": dict(T=4096, E=128, K=8, D=4096, H=1536, O=4096, kind="swiglu", dtype="fp8", routing="uniform"),
+}
+
+
+def flops_of(w):
+    R = w["T"] * w["K"]
+    hn = 2 * w["H"] if w["kind"] == "swiglu" else w["H"]
+    return 2.0 * R * w["D"] * hn, 2.0 * R * w["H"] * w["O"]
+
+
+def make_inputs(w, device, seed=0):
+    """Synthetic tensors of the workload's shape, generated on `device`."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    bf = torch.bfloat16
+    T, E, K, D, H, O = (w[k] for k in "TEKDHO")
+    rn = lambda *s: torch.randn(*s, generator=g, device=device)
+    x = rn(T, D).to(bf)
+    if w["dtype"] == "fp8":          # 1 % of the token rows scaled x100 as outliers
+        rows = torch.randperm(T, generator=g, device=device)[: max(1, T // 100)]
+        x[rows] = (x[rows].float() * 100).to(bf)
+    inp = {"x": x}
+    if w["kind"] == "swiglu":
+        inp["w_gate"] = (rn(E, H, D) * D ** -0.5).to(bf)     # stored [E, N, K], passed as [E, K, N] views
+        inp["w_up"] = (rn(E, H, D) * D ** -0.5).to(bf)
+        inp["w_down"] = (rn(E, O, H) * H ** -0.5).to(bf)
+    else:
+        inp["w1"] = (rn(E, H, D) * D ** -0.5).to(bf)
+        inp["b1"] = torch.zeros(E, H, dtype=bf, device=device)
+        inp["w2"] = (rn(E, O, H) * H ** -0.5).to(bf)
+        inp["b2"] = torch.zeros(E, O, dtype=bf, device=device)
+    w_gate_net = rn(D, E) * D ** -0.5
+    logits = x.float() @ w_gate_net
+    if w["routing"] == "zipf":       # per-expert Zipf(1.1) bias; the last two experts get no token
+        p = (torch.arange(E, device=device, dtype=torch.float32) + 1) ** -1.1
+        logits = logits + torch.log(p / p.sum())
+        logits[:, E - 2:] = -1e30
+    elif w["routing"] == "uniform":  # uniform random distinct experts, gates 1/K after renormalisation
+        logits = torch.rand(T, E, generator=g, device=device) * 1e-3
+    scores = torch.softmax(logits, dim=1)
+    inp["scores"] = scores if w["kind"] == "swiglu" else scores.to(bf)
+    return inp
+
+
+class GpuPath:
+    """The hot path through the library, split into its kernels so that each can be timed."""
+
+    def __init__(self, w, inp):
+        from fast_moe_amd.kernels import moe_fp8
+        from fast_moe_amd.kernels.hip import ops
+        self.ops, self.w, self.inp = ops, w, inp
+        self.fp8 = w["dtype"] == "fp8"
+        v = lambda t: t.permute(0, 2, 1)
+        if w["kind"] == "swiglu":
+            self.wg, self.wu, self.wd = v(inp["w_gate"]), v(inp["w_up"]), v(inp["w_down"])
+            if self.fp8:             # weights are quantised once, outside the step
+                self.qg, self.sg = moe_fp8.quantize_expert_weights(self.wg)
+                self.qu, self.su = moe_fp8.quantize_expert_weights(self.wu)
+                self.qd, self.sd = moe_fp8.quantize_expert_weights(self.wd)
+        else:
+            self.w1, self.w2 = v(inp["w1"]), v(inp["w2"])
+
+    # --- the pieces
+    def route(self):
+        self.r = self.ops.route_topk(self.inp["scores"], self.w["K"])
+        return self.r
+
+    def quant_tokens(self):
+        self.qx, self.sx = self.ops.quant_rows_fp8(self.inp["x"])
+
+    def gemm1(self):
+        o, w, r, K = self.ops, self.w, self.r, self.w["K"]
+        R = w["T"] * K
+        if w["kind"] == "mlp":
+            self.hidden = o.grouped_gemm(r["offsets"], self.inp["x"], self.w1, total_rows=R,
+                                         row_index=r["gate_index"], index_div=K, bias=self.inp["b1"], epilogue=1)
+        elif self.fp8:
+            self.hidden = o.grouped_gemm(r["offsets"], self.qx, self.qg, total_rows=R, row_index=r["gate_index"],
+                                         index_div=K, b2=self.qu, epilogue=2, a_scale=self.sx, b_scale=self.sg,
+                                         b2_scale=self.su)
+        else:
+            self.hidden = o.grouped_gemm(r["offsets"], self.inp["x"], self.wg, total_rows=R,
+                                         row_index=r["gate_index"], index_div=K, b2=self.wu, epilogue=2)
+
+    def quant_hidden(self):
+        self.qh, self.sh = self.ops.quant_rows_fp8(self.hidden)
+
+    def gemm2(self):
+        o, r = self.ops, self.r
+        R = self.w["T"] * self.w["K"]
+        if self.w["kind"] == "mlp":
+            self.rows = o.grouped_gemm(r["offsets"], self.hidden, self.w2, total_rows=R, bias=self.inp["b2"])
+        elif self.fp8:
+            self.rows = o.grouped_gemm(r["offsets"], self.qh, self.qd, total_rows=R, a_scale=self.sh,
+                                       b_scale=self.sd)
+        else:
+            self.rows = o.grouped_gemm(r["offsets"], self.hidden, self.wd, total_rows=R)
+
+    def combine(self):
+        r = self.r
+        gates = r["gates"] if self.w["kind"] == "mlp" else r["gates"].to(torch.bfloat16)
+        self.y = self.ops.combine(self.rows, r["reverse_index"], gates, r["gate_index"])
+        return self.y
+
+    def pieces(self):
+        seq = [("route", self.route)]
+        if self.fp8:
+            seq.append(("quant_tokens", self.quant_tokens))
+        seq.append(("gemm1", self.gemm1))
+        if self.fp8:
+            seq.append(("quant_hidden", self.quant_hidden))
+        seq += [("gemm2", self.gemm2), ("combine", self.combine)]
+        return seq
+
+    def step(self):
+        for _, fn in self.pieces():
+            fn()
+        return self.y
+
+
+def time_region(fn, iters, stream):
+    """Average milliseconds of `fn` over `iters` launches, HIP events on the launch stream."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for _ in range(iters):
+        fn()
+    stop.record(stream)
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def algorithmic_bytes(w, name):
+    T, E, K, D, H, O = (w[k] for k in "TEKDHO")
+    R = T * K
+    if name == "route":
+        sb = 2 if w["kind"] == "mlp" else 4
+        return T * E * sb + 3 * R * 8 + T * K * (8 + sb) + (2 * E + 1) * 8
+    if name == "quant_tokens":
+        return T * D * 3 + T * 4
+    if name == "quant_hidden":
+        return R * H * 3 + R * 4
+    if name == "combine":
+        return R * O * 2 + T * O * 2 + R * (8 + 8 + 2)
+    return None
+
+
+def run_gpu(w, steps, warmup):
+    dev = torch.device("cuda:0")
+    inp = make_inputs(w, dev)
+    path = GpuPath(w, inp)
+    stream = torch.cuda.current_stream(dev)
+    for _ in range(max(warmup, 1)):
+        path.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        path.step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / steps
+    # per-kernel launch durations, measured live with events over the same number of launches
+    path.step()
+    per = {}
+    for name, fn in path.pieces():
+        torch.cuda.synchronize()
+        per[name] = time_region(fn, steps, stream)
+    f1, f2 = flops_of(w)
+    kernels = {}
+    for name, ms in per.items():
+        entry = {"ms": round(ms, 4)}
+        if name == "gemm1":
+            entry["tflops"] = round(f1 / ms / 1e9, 1)
+        elif name == "gemm2":
+            entry["tflops"] = round(f2 / ms / 1e9, 1)
+        else:
+            b = algorithmic_bytes(w, name)
+            if b:
+                entry["gbs"] = round(b / ms / 1e6, 1)
+        kernels[name] = entry
+    lengths = path.r["lengths"]
+    stats = {"rows_max": int(lengths.max()), "rows_min": int(lengths.min()),
+             "empty_experts": int((lengths == 0).sum())}
+    return ms_step, kernels, stats, (f1, f2)
+
+
+def cpu_baseline(w, budget_s=12.0):
+    """The oracle (CPU restatement of the reference's PyTorch path) on a bounded sample of the
+    same workload: same dims and routing law, fewer tokens."""
+    from oracle import layer as o_layer
+    from oracle import moe as o_moe
+    from oracle import moe_fp8 as o_fp8
+    cores = torch.get_num_threads()
+    sample_T = 256
+    result = None
+    while True:
+        ws = dict(w, T=sample_T)
+        inp = make_inputs(ws, torch.device("cpu"), seed=1)
+        K = w["K"]
+        v = lambda t: t.permute(0, 2, 1)
+
+        def run():
+            r = o_layer.route_scores(inp["scores"], K)
+            idx2 = r["gate_index"].view(-1, K)
+            if w["kind"] == "mlp":
+                h = o_moe.index_select_jagged_bmm(r["offsets"], idx2, inp["x"], v(inp["w1"]), inp["b1"])
+                return o_moe.silu_jagged_bmm_combine(r["offsets"], h, v(inp["w2"]), inp["b2"], r["token_index"], K,
+                                                     r["gates"], r["gate_index"])
+            gates = r["gates"].to(torch.bfloat16)
+            if w["dtype"] == "fp8":
+                return o_fp8.swiglu_moe_fp8(r["offsets"], idx2, inp["x"], v(inp["w_gate"]), None, v(inp["w_up"]),
+                                            None, v(inp["w_down"]), None, r["token_index"], K, gates,
+                                            r["gate_index"])[0]
+            return o_moe.fused_jagged_bmm_swiglu_combine(r["offsets"], idx2, inp["x"], v(inp["w_gate"]), None,
+                                                         v(inp["w_up"]), None, v(inp["w_down"]), None, K, gates,
+                                                         r["gate_index"])
+
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        f1, f2 = flops_of(ws)
+        result = {"value": round((f1 + f2) / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                  "sample": f"oracle PyTorch-kernel path, {w['dtype']} emulation, T={sample_T} of {w['T']} tokens "
+                            f"(same E/K/D/H, same routing law), 1 pass, {dt:.1f} s",
+                  "tokens_per_s": round(sample_T / dt, 1)}
+        if dt * 4 > budget_s or sample_T * 4 > w["T"]:
+            return result
+        sample_T *= 4
+
+
+def bench_workload(name, steps, warmup, tokens=None):
+    w = dict(WORKLOADS[name])
+    if tokens:
+        w["T"] = tokens
+    ms, kernels, stats, (f1, f2) = run_gpu(w, steps, warmup)
+    return w, ms, kernels, stats, f1 + f2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c3_bf16", choices=sorted(WORKLOADS))
+    ap.add_argument("--tokens", type=int, default=None, help="override the token count (C5 sweep)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary fp8 / bf16 workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU with all experts local; expert parallelism is out of "
+              "scope, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    w, ms, kernels, stats, flops = bench_workload(args.workload, args.steps, args.warmup, args.tokens)
+    dt = w["dtype"]
+    g1 = kernels["gemm1"]
+    line = {
+        "metric": "moe_forward_tflops", "value": round(flops / ms / 1e9, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if dt == "bf16" else "fp8_e4m3", "data": "synthetic",
+        "tokens_per_s": round(w["T"] / ms * 1e3, 1),
+        "config": {"workload": f"{args.workload}: {w['kind']} MoE forward, T={w['T']} tokens, E={w['E']} experts, "
+                               f"top-{w['K']}, D={w['D']}, H={w['H']}, O={w['O']}, routing={w['routing']}",
+                   "tokens": w["T"], "experts": w["E"], "top_k": w["K"], "d_model": w["D"], "hidden": w["H"],
+                   "routing": stats},
+        "kernels": kernels,
+        "roofline": {"bound": "mfma", "kernel": "grouped_gemm (gemm1: gather + GEMM + " +
+                     ("SwiGLU" if w["kind"] == "swiglu" else "SiLU") + " epilogue)",
+                     "achieved": g1["tflops"], "peak": PEAK[dt], "unit": "TFLOP/s",
+                     "frac": round(g1["tflops"] / PEAK[dt], 4), "traffic": None},
+    }
+    if not args.no_extra:
+        other = {"c3_bf16": "c4_fp8", "c4_fp8": "c3_bf16"}.get(args.workload)
+        if other:
+            w2, ms2, k2, _, fl2 = bench_workload(other, args.steps, args.warmup)
+            line["extra"] = {other: {"value": round(fl2 / ms2 / 1e9, 2), "unit": "TFLOP/s",
+                                     "ms_per_step": round(ms2, 4), "tokens_per_s": round(w2["T"] / ms2 * 1e3, 1),
+                                     "kernels": k2}}
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,176 @@
+// Weighted merge of the K expert rows of every token (gather form, no atomics):
+// each output row is produced by exactly one wavefront that adds its K source
+// rows in ascending source-row order, which is the order of a sequential
+// index_add and therefore reproducible bit for bit.
+#include "common.h"
+
+namespace fmoe {
+namespace {
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+    static constexpr int kVec = 4;
+    __device__ static float load(const float* p) { return *p; }
+    __device__ static void store(float* p, float v) { *p = v; }
+    __device__ static void unpack(const u32x4& raw, float* f) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(raw[i]);
+    }
+    __device__ static u32x4 pack(const float* f) {
+        return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+                     __float_as_uint(f[3])};
+    }
+};
+template <>
+struct Elem<uint16_t> {
+    static constexpr int kVec = 8;
+    __device__ static float load(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+    __device__ static void store(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
+    __device__ static void unpack(const u32x4& raw, float* f) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = bf16_bits_to_f32(raw[i] & 0xffffu);
+            f[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+        }
+    }
+    __device__ static u32x4 pack(const float* f) {
+        u32x4 r;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = f32_to_bf16_bits(f[2 * i]) | (f32_to_bf16_bits(f[2 * i + 1]) << 16);
+        return r;
+    }
+};
+
+struct GateView {
+    const void* ptr;
+    int64_t cols, stride_row, stride_col;
+    const int64_t* index;
+    int64_t numel;
+};
+
+template <typename TG>
+__device__ __forceinline__ float gate_of(const GateView& g, int64_t r, bool& ok) {
+    int64_t flat = g.index ? g.index[r] : r;
+    ok = (uint64_t)flat < (uint64_t)g.numel;
+    if (!ok) return 0.0f;
+    const int64_t gr = flat / g.cols, gc = flat - gr * g.cols;
+    return Elem<TG>::load((const TG*)g.ptr + gr * g.stride_row + gc * g.stride_col);
+}
+
+// TV value dtype, TG gate dtype, ROUND_BF16: the product is rounded to bf16
+// (both operands bf16); HAS_GATE false = plain segmented sum.
+// VECTOR: 16-byte loads, one wave covers 64*kVec columns of one token.
+template <typename TV, typename TG, typename TO, bool HAS_GATE, bool ROUND_BF16, bool VECTOR>
+__global__ __launch_bounds__(256) void combine_kernel(const TV* __restrict__ value, int64_t T, int K,
+                                                      int64_t D, int64_t stride_row,
+                                                      const int64_t* __restrict__ reverse_index,
+                                                      GateView gate, TO* __restrict__ out,
+                                                      int chunks_per_token) {
+    constexpr int VEC = VECTOR ? Elem<TV>::kVec : 1;
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
+    const int64_t t = wave / chunks_per_token;
+    const int chunk = (int)(wave - t * chunks_per_token);
+    if (t >= T) return;
+    const int64_t col = ((int64_t)chunk * kWave + lane) * VEC;
+    const bool active = col < D;
+    const int64_t R = T * K;
+    float acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
+#pragma unroll 4
+    for (int j = 0; j < K; ++j) {
+        const int64_t r = reverse_index[t * K + j];
+        if ((uint64_t)r >= (uint64_t)R) continue;       // malformed index: contributes nothing
+        float w = 1.0f;
+        if (HAS_GATE) {
+            bool ok;
+            w = gate_of<TG>(gate, r, ok);
+            if (!ok) continue;
+        }
+        if (!active) continue;
+        float f[VEC];
+        if (VECTOR) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(value + r * stride_row + col);
+            Elem<TV>::unpack(raw, f);
+        } else {
+            f[0] = Elem<TV>::load(value + r * stride_row + col);
+        }
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+            float p = HAS_GATE ? f[i] * w : f[i];
+            if (HAS_GATE && ROUND_BF16) p = round_bf16(p);
+            acc[i] = acc[i] + p;
+        }
+    }
+    if (!active) return;
+    if (VECTOR && sizeof(TO) == sizeof(TV)) {
+        *reinterpret_cast<u32x4*>(out + t * D + col) = Elem<TO>::pack(acc);
+    } else {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) Elem<TO>::store(out + t * D + col + i, acc[i]);
+    }
+}
+
+template <typename TV, typename TG, typename TO, bool HAS_GATE, bool ROUND_BF16>
+void launch(const void* value, int64_t T, int K, int64_t D, int64_t stride_row,
+            const int64_t* reverse_index, const GateView& gate, void* out, hipStream_t stream) {
+    constexpr int vec = Elem<TV>::kVec;
+    const bool vector = (D % vec) == 0 && (stride_row % vec) == 0 && aligned16(value) && aligned16(out);
+    const int per_wave = kWave * (vector ? vec : 1);
+    const int chunks = (int)((D + per_wave - 1) / per_wave);
+    const int64_t waves = T * chunks;
+    const unsigned blocks = (unsigned)((waves + 3) / 4);
+    if (vector)
+        combine_kernel<TV, TG, TO, HAS_GATE, ROUND_BF16, true><<<blocks, 256, 0, stream>>>(
+            (const TV*)value, T, K, D, stride_row, reverse_index, gate, (TO*)out, chunks);
+    else
+        combine_kernel<TV, TG, TO, HAS_GATE, ROUND_BF16, false><<<blocks, 256, 0, stream>>>(
+            (const TV*)value, T, K, D, stride_row, reverse_index, gate, (TO*)out, chunks);
+}
+
+}  // namespace
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" int fmoe_combine(const void* value, int value_dtype, int64_t T, int K, int64_t D,
+                            int64_t value_stride_row, const int64_t* reverse_index, const void* gates,
+                            int gates_dtype, int64_t gates_cols, int64_t gates_stride_row,
+                            int64_t gates_stride_col, const int64_t* gates_index, void* out, int out_dtype,
+                            fmoe_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    FMOE_REQUIRE(T >= 0 && K >= 1 && D >= 1, "fmoe_combine: need T >= 0, K >= 1, D >= 1");
+    FMOE_REQUIRE(value_dtype == FMOE_BF16 || value_dtype == FMOE_F32, "fmoe_combine: value must be bf16 or fp32");
+    if (T == 0) return FMOE_OK;
+    FMOE_REQUIRE(value && reverse_index && out, "fmoe_combine: NULL pointer");
+    FMOE_REQUIRE(value_stride_row >= D, "fmoe_combine: value row stride %lld < D %lld",
+                 (long long)value_stride_row, (long long)D);
+    FMOE_REQUIRE(T * (int64_t)((D + 63) / 64) < ((int64_t)1 << 33), "fmoe_combine: problem too large");
+    GateView g{gates, gates_cols, gates_stride_row, gates_stride_col, gates_index, T * (int64_t)K};
+    int expect_out = value_dtype;
+    if (gates) {
+        FMOE_REQUIRE(gates_dtype == FMOE_BF16 || gates_dtype == FMOE_F32, "fmoe_combine: gates must be bf16 or fp32");
+        FMOE_REQUIRE(gates_cols >= 1, "fmoe_combine: gates_cols < 1");
+        if (gates_dtype == FMOE_F32) expect_out = FMOE_F32;
+    }
+    FMOE_REQUIRE(out_dtype == expect_out,
+                 "fmoe_combine: out dtype must be the promoted dtype of value and gates (%d), got %d",
+                 expect_out, out_dtype);
+    const bool vb = value_dtype == FMOE_BF16;
+    if (!gates) {
+        if (vb) launch<uint16_t, float, uint16_t, false, false>(value, T, K, D, value_stride_row, reverse_index, g, out, stream);
+        else launch<float, float, float, false, false>(value, T, K, D, value_stride_row, reverse_index, g, out, stream);
+    } else if (vb && gates_dtype == FMOE_BF16) {
+        launch<uint16_t, uint16_t, uint16_t, true, true>(value, T, K, D, value_stride_row, reverse_index, g, out, stream);
+    } else if (vb) {
+        launch<uint16_t, float, float, true, false>(value, T, K, D, value_stride_row, reverse_index, g, out, stream);
+    } else if (gates_dtype == FMOE_BF16) {
+        launch<float, uint16_t, float, true, false>(value, T, K, D, value_stride_row, reverse_index, g, out, stream);
+    } else {
+        launch<float, float, float, true, false>(value, T, K, D, value_stride_row, reverse_index, g, out, stream);
+    }
+    return check_launch("fmoe_combine");
+}

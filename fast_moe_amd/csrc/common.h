@@ -1,0 +1,90 @@
+// Shared host/device helpers for the gfx950 kernels of libfastmoe_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/fast_moe_amd.h"
+
+namespace fmoe {
+
+// ---------------------------------------------------------------- host side
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+#define FMOE_REQUIRE(cond, ...)                                   \
+    do {                                                          \
+        if (!(cond)) return ::fmoe::fail(FMOE_ERR_ARGUMENT, __VA_ARGS__); \
+    } while (0)
+
+__host__ __device__ static inline bool aligned16(const void* p) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+__host__ __device__ static inline bool aligned_ok(const void* a, const void* b, const void* c) {
+    return aligned16(a) && aligned16(b) && aligned16(c);
+}
+
+// -------------------------------------------------------------- device side
+constexpr int kWave = 64;
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bit pattern; NaN stays NaN (quiet)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+// SiLU from the hardware exp / reciprocal (about 2 ulp in fp32): for values that
+// are rounded to bf16 right afterwards.
+__device__ __forceinline__ float fast_silu_f32(float x) { return __fdividef(x, 1.0f + __expf(-x)); }
+
+__device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
+template <typename T>
+__device__ __forceinline__ T wave_bcast(T v, int src_lane) {
+    return __shfl(v, src_lane, kWave);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// inclusive prefix sum over the 64 lanes
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        int n = __shfl_up(v, o, kWave);
+        if (lane >= o) v += n;
+    }
+    return v;
+}
+__device__ __forceinline__ long long wave_inclusive_scan(long long v) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        long long n = __shfl_up(v, o, kWave);
+        if (lane >= o) v += n;
+    }
+    return v;
+}
+
+}  // namespace fmoe

@@ -1,0 +1,82 @@
+// Error reporting, version, and the small element-wise kernel of libfastmoe_hip.so.
+#include "common.h"
+
+#include <cstring>
+
+namespace fmoe {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_launch(const char* what) {
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return fail(FMOE_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(err));
+    return FMOE_OK;
+}
+
+namespace {
+
+// out = round(round(silu(a)) * b), 8 bf16 per thread
+__global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __restrict__ a,
+                                                            const uint16_t* __restrict__ b,
+                                                            uint16_t* __restrict__ out, int64_t n) {
+    const int64_t i0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i0 + 8 <= n && aligned_ok(a, b, out)) {
+        const u32x4 va = *reinterpret_cast<const u32x4*>(a + i0);
+        const u32x4 vb = *reinterpret_cast<const u32x4*>(b + i0);
+        u32x4 vo;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t r = 0;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const float x = bf16_bits_to_f32((va[j] >> (16 * h)) & 0xffffu);
+                const float y = bf16_bits_to_f32((vb[j] >> (16 * h)) & 0xffffu);
+                r |= f32_to_bf16_bits(round_bf16(silu_f32(x)) * y) << (16 * h);
+            }
+            vo[j] = r;
+        }
+        *reinterpret_cast<u32x4*>(out + i0) = vo;
+    } else {
+        for (int64_t i = i0; i < n && i < i0 + 8; ++i) {
+            const float x = bf16_bits_to_f32(a[i]);
+            const float y = bf16_bits_to_f32(b[i]);
+            out[i] = (uint16_t)f32_to_bf16_bits(round_bf16(silu_f32(x)) * y);
+        }
+    }
+}
+
+}  // namespace
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" int fmoe_version(void) { return 100; }
+
+extern "C" const char* fmoe_last_error(void) { return g_error; }
+
+extern "C" int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
+                             fmoe_stream_t stream) {
+    FMOE_REQUIRE(dtype == FMOE_BF16, "fmoe_silu_mul: only bf16 is supported");
+    FMOE_REQUIRE(n >= 0, "fmoe_silu_mul: n < 0");
+    if (n == 0) return FMOE_OK;
+    FMOE_REQUIRE(a && b && out, "fmoe_silu_mul: NULL pointer");
+    const int64_t threads = (n + 7) / 8;
+    silu_mul_bf16_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, n);
+    return check_launch("fmoe_silu_mul");
+}

@@ -1,0 +1,74 @@
+// fmoe_grouped_gemm: argument checks and kernel selection for the jagged GEMM.
+#include "gemm_kernel.h"
+
+using namespace fmoe;
+
+extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    FMOE_REQUIRE(d != nullptr, "fmoe_grouped_gemm: desc is NULL");
+    FMOE_REQUIRE(d->num_experts >= 1 && d->n >= 1 && d->k >= 1,
+                 "fmoe_grouped_gemm: need E, n, k >= 1 (E=%d n=%d k=%d)", d->num_experts, d->n, d->k);
+    FMOE_REQUIRE(d->total_rows >= 0, "fmoe_grouped_gemm: total_rows < 0");
+    FMOE_REQUIRE(d->a_dtype == FMOE_BF16 || d->a_dtype == FMOE_E4M3,
+                 "fmoe_grouped_gemm: operands must be bf16 or e4m3 (got dtype %d)", d->a_dtype);
+    FMOE_REQUIRE(d->out_dtype == FMOE_BF16, "fmoe_grouped_gemm: output must be bf16");
+    FMOE_REQUIRE(d->epilogue >= FMOE_EPI_NONE && d->epilogue <= FMOE_EPI_SWIGLU,
+                 "fmoe_grouped_gemm: unknown epilogue %d", d->epilogue);
+    if (d->total_rows == 0) return FMOE_OK;
+    FMOE_REQUIRE(d->offsets && d->a && d->b && d->out, "fmoe_grouped_gemm: NULL tensor pointer");
+    FMOE_REQUIRE(d->a_rows >= 1, "fmoe_grouped_gemm: a_rows < 1");
+    FMOE_REQUIRE(d->index_div >= 1, "fmoe_grouped_gemm: index_div < 1");
+    FMOE_REQUIRE(d->a_stride_row >= d->k, "fmoe_grouped_gemm: A row stride %lld < k %d",
+                 (long long)d->a_stride_row, d->k);
+    FMOE_REQUIRE(d->out_stride_row >= d->n, "fmoe_grouped_gemm: out row stride %lld < n %d",
+                 (long long)d->out_stride_row, d->n);
+    const bool fp8 = d->a_dtype == FMOE_E4M3;
+    const bool swiglu = d->epilogue == FMOE_EPI_SWIGLU;
+    if (swiglu) FMOE_REQUIRE(d->b2 != nullptr, "fmoe_grouped_gemm: SWIGLU needs b2");
+    if (fp8) {
+        FMOE_REQUIRE(d->a_scale && d->b_scale, "fmoe_grouped_gemm: e4m3 operands need a_scale and b_scale");
+        if (swiglu) FMOE_REQUIRE(d->b2_scale != nullptr, "fmoe_grouped_gemm: SWIGLU e4m3 needs b2_scale");
+        FMOE_REQUIRE(!d->a_silu, "fmoe_grouped_gemm: a_silu is not defined for e4m3 operands");
+    }
+
+    GemmParams p;
+    p.offsets = d->offsets;
+    p.row_index = d->row_index;
+    p.E = d->num_experts;
+    p.N = d->n;
+    p.K = d->k;
+    p.index_div = d->index_div;
+    p.total_rows = d->total_rows;
+    p.a_rows = d->a_rows;
+    p.a = (const uint8_t*)d->a;
+    p.a_stride_row = d->a_stride_row;
+    p.a_stride_e = d->a_stride_e;
+    p.a_scale = d->a_scale;
+    p.b = (const uint8_t*)d->b;
+    p.b2 = (const uint8_t*)d->b2;
+    p.b_se = d->b_stride_e;
+    p.b_sk = d->b_stride_k;
+    p.b_sn = d->b_stride_n;
+    p.b_scale = d->b_scale;
+    p.b2_scale = d->b2_scale;
+    p.bias = (const uint16_t*)d->bias;
+    p.bias2 = (const uint16_t*)d->bias2;
+    p.bias_se = d->bias_stride_e;
+    p.out = (uint16_t*)d->out;
+    p.out_stride = d->out_stride_row;
+    p.n_tiles = 0;
+    p.vec_store = (d->n % 4 == 0) && (d->out_stride_row % 4 == 0) &&
+                  ((reinterpret_cast<uintptr_t>(d->out) & 7u) == 0);
+
+    const int esize = fp8 ? 1 : 2;
+    const int chunk = 16 / esize;
+    const bool fast = d->b_stride_k == 1 && (d->k % chunk) == 0 && aligned16(d->a) && aligned16(d->b) &&
+                      (!swiglu || aligned16(d->b2)) && (d->a_stride_row % chunk) == 0 &&
+                      (d->a_stride_e % chunk) == 0 && (d->b_stride_n % chunk) == 0 &&
+                      (d->b_stride_e % chunk) == 0;
+    // rows per expert decide the tile height: tall tiles for prefill-like loads,
+    // short ones when the experts see a handful of rows (weight-streaming regime)
+    const bool big = d->total_rows / d->num_experts >= 96;
+    if (fp8) return run_gemm_fp8(p, d->epilogue, fast, big, stream);
+    return run_gemm_bf16(p, d->epilogue, d->a_silu != 0, fast, big, stream);
+}

@@ -1,0 +1,17 @@
+// OCP e4m3 instantiations of the jagged GEMM (v_mfma_f32_32x32x64_f8f6f4, both
+// operand formats = e4m3, unit block scales; the row-wise power-of-two scales
+// are divided out in the epilogue).
+#include "gemm_kernel.h"
+
+namespace fmoe {
+
+int run_gemm_fp8(GemmParams& p, int epilogue, bool fast, bool big, hipStream_t stream) {
+    switch (epilogue) {
+        case FMOE_EPI_NONE: return dispatch_tile<true, FMOE_EPI_NONE, false>(p, fast, big, stream);
+        case FMOE_EPI_SILU: return dispatch_tile<true, FMOE_EPI_SILU, false>(p, fast, big, stream);
+        case FMOE_EPI_SWIGLU: return dispatch_tile<true, FMOE_EPI_SWIGLU, false>(p, fast, big, stream);
+    }
+    return fail(FMOE_ERR_ARGUMENT, "fmoe_grouped_gemm: unknown epilogue %d", epilogue);
+}
+
+}  // namespace fmoe

@@ -1,0 +1,404 @@
+// Routing for the MoE forward: top-k selection with L1-renormalised gates, the
+// per-expert histogram / prefix sum ("jagged offsets") and the stable
+// expert-major permutation with its inverse.  All integer outputs are a pure
+// function of the selected ids (a stable counting sort), so they are
+// reproducible bit for bit.
+//
+// Pipeline (4 launches on one stream, no host synchronisation):
+//   1. topk_kernel     rank-by-counting selection, one token per LPT lanes
+//   2. hist_kernel     one wave per chunk of tokens: LDS histogram -> chunk_hist[c][e]
+//   3. scan_kernel     one block: exclusive scan of chunk_hist over chunks (in
+//                      place), lengths[e], offsets[e] (wave scan over experts)
+//   4. scatter_kernel  one wave per chunk: wave-level match/rank gives each
+//                      position its slot inside its expert segment
+#include "common.h"
+
+namespace fmoe {
+namespace {
+
+constexpr int kMaxChunks = 512;
+constexpr int kScanThreads = 1024;
+constexpr uint16_t kBadExpert = 0xFFFF;
+
+struct RoutePlan {
+    int64_t tokens_per_chunk;
+    int num_chunks;
+    size_t compact_bytes;   // uint16 expert id per routed position
+    size_t hist_bytes;      // int32 [num_chunks][E]
+    size_t total_bytes;
+};
+
+RoutePlan make_plan(int64_t T, int E, int K) {
+    RoutePlan p;
+    p.tokens_per_chunk = (T + kMaxChunks - 1) / kMaxChunks;
+    if (p.tokens_per_chunk < 1) p.tokens_per_chunk = 1;
+    p.num_chunks = (int)((T + p.tokens_per_chunk - 1) / p.tokens_per_chunk);
+    if (p.num_chunks < 1) p.num_chunks = 1;
+    size_t compact = (size_t)T * (size_t)K * sizeof(uint16_t);
+    p.compact_bytes = (compact + 255) & ~(size_t)255;
+    p.hist_bytes = ((size_t)p.num_chunks * (size_t)E * sizeof(int32_t) + 255) & ~(size_t)255;
+    p.total_bytes = p.compact_bytes + p.hist_bytes + 256;
+    return p;
+}
+
+template <typename T>
+__device__ __forceinline__ float load_score(const T* p);
+template <>
+__device__ __forceinline__ float load_score<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float load_score<uint16_t>(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+
+template <typename T>
+__device__ __forceinline__ float round_to(float v);
+template <>
+__device__ __forceinline__ float round_to<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float round_to<uint16_t>(float v) { return round_bf16(v); }
+
+template <typename T>
+__device__ __forceinline__ void store_score(T* p, float v);
+template <>
+__device__ __forceinline__ void store_score<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void store_score<uint16_t>(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
+
+// One token per LPT lanes, VPL scores per lane (expert id = v*LPT + sub).  The
+// rank of a score is the number of scores that beat it (greater, or equal with
+// a lower expert id); rank < K selects it and is its slot.
+template <typename T, int LPT, int VPL>
+__global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores, int64_t num_tokens,
+                                                   int E, int K, int renorm,
+                                                   int64_t* __restrict__ topk_idx,
+                                                   T* __restrict__ gates,
+                                                   uint16_t* __restrict__ compact) {
+    constexpr int TPW = kWave / LPT;          // tokens per wave
+    constexpr int WPB = 256 / kWave;
+    __shared__ float s_sel[WPB][TPW][64];     // selected scores by slot (K <= 64)
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    const int sub = lane % LPT;
+    const int grp = lane / LPT;
+    const int64_t t = ((int64_t)blockIdx.x * WPB + wave) * TPW + grp;
+    const bool live = t < num_tokens;
+
+    float my[VPL];
+    const float ninf = -__builtin_inff();
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = v * LPT + sub;
+        my[v] = (live && e < E) ? load_score<T>(scores + t * E + e) : ninf;
+    }
+    int rank[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) rank[v] = 0;
+#pragma unroll
+    for (int u = 0; u < VPL; ++u) {
+#pragma unroll 8
+        for (int i = 0; i < LPT; ++i) {
+            const float other = __shfl(my[u], grp * LPT + i, kWave);
+            const int oe = u * LPT + i;
+#pragma unroll
+            for (int v = 0; v < VPL; ++v) {
+                const int e = v * LPT + sub;
+                rank[v] += (other > my[v] || (other == my[v] && oe < e)) ? 1 : 0;
+            }
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = v * LPT + sub;
+        if (live && e < E && rank[v] < K) s_sel[wave][grp][rank[v]] = my[v];
+    }
+    __syncthreads();
+    if (!live) return;
+    float denom = 1.0f;
+    if (renorm) {
+        float s = 0.0f;
+        for (int j = 0; j < K; ++j) s = s + fabsf(s_sel[wave][grp][j]);   // slot order
+        denom = fmaxf(round_to<T>(s), round_to<T>(1e-12f));
+    }
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = v * LPT + sub;
+        if (e < E && rank[v] < K) {
+            const int64_t p = t * K + rank[v];
+            topk_idx[p] = e;
+            compact[p] = (uint16_t)e;
+            store_score<T>(gates + p, renorm ? round_to<T>(my[v] / denom) : my[v]);
+        }
+    }
+}
+
+// Expert ids supplied by the caller (int64): narrow to the compact form, flag
+// out-of-range ids.
+__global__ __launch_bounds__(256) void compact_kernel(const int64_t* __restrict__ topk_idx, int64_t n,
+                                                      int E, uint16_t* __restrict__ compact,
+                                                      int64_t* __restrict__ bad_count) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t e = topk_idx[i];
+    const bool ok = e >= 0 && e < E;
+    compact[i] = ok ? (uint16_t)e : kBadExpert;
+    if (!ok && bad_count) atomicAdd((unsigned long long*)bad_count, 1ull);
+}
+
+__global__ void zero_i64_kernel(int64_t* p) { *p = 0; }
+
+// One wave per chunk of tokens; counts are integers, so LDS atomics are exact.
+__global__ __launch_bounds__(kWave) void hist_kernel(const uint16_t* __restrict__ compact,
+                                                     int64_t total_pos, int64_t pos_per_chunk, int E,
+                                                     int32_t* __restrict__ chunk_hist) {
+    extern __shared__ int32_t s_cnt[];
+    const int c = blockIdx.x;
+    for (int e = threadIdx.x; e < E; e += kWave) s_cnt[e] = 0;
+    __syncthreads();
+    const int64_t begin = (int64_t)c * pos_per_chunk;
+    int64_t end = begin + pos_per_chunk;
+    if (end > total_pos) end = total_pos;
+    for (int64_t p = begin + threadIdx.x; p < end; p += kWave) {
+        const uint16_t e = compact[p];
+        if (e != kBadExpert) atomicAdd(&s_cnt[e], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += kWave) chunk_hist[(int64_t)c * E + e] = s_cnt[e];
+}
+
+// Single block.  Threads form [SEG][EW] (EW = power of two >= E): thread (s, e)
+// owns chunks [s*cps, (s+1)*cps) of expert e.
+__global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict__ chunk_hist,
+                                                            int num_chunks, int E, int EW,
+                                                            int64_t* __restrict__ lengths,
+                                                            int64_t* __restrict__ offsets) {
+    extern __shared__ int32_t s_buf[];   // [SEG][EW] partials, then [E] totals
+    const int SEG = kScanThreads / EW;
+    const int e = threadIdx.x % EW;
+    const int s = threadIdx.x / EW;
+    const int cps = (num_chunks + SEG - 1) / SEG;
+    const int c0 = s * cps;
+    int c1 = c0 + cps;
+    if (c1 > num_chunks) c1 = num_chunks;
+    int32_t part = 0;
+    if (e < E)
+        for (int c = c0; c < c1; ++c) part += chunk_hist[(int64_t)c * E + e];
+    s_buf[s * EW + e] = part;
+    __syncthreads();
+    int32_t base = 0, total = 0;
+    for (int q = 0; q < SEG; ++q) {
+        const int32_t v = s_buf[q * EW + e];
+        if (q < s) base += v;
+        total += v;
+    }
+    if (e < E) {
+        int32_t run = base;
+        for (int c = c0; c < c1; ++c) {
+            const int64_t i = (int64_t)c * E + e;
+            const int32_t v = chunk_hist[i];
+            chunk_hist[i] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    int32_t* s_tot = s_buf;
+    if (s == 0 && e < E) {
+        s_tot[e] = total;
+        lengths[e] = total;
+    }
+    __syncthreads();
+    if (threadIdx.x < kWave) {
+        long long run = 0;
+        if (threadIdx.x == 0) offsets[0] = 0;
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int ee = e0 + threadIdx.x;
+            const long long v = ee < E ? (long long)s_tot[ee] : 0;
+            const long long inc = wave_inclusive_scan(v);
+            if (ee < E) offsets[ee + 1] = run + inc;
+            run += wave_bcast(inc, kWave - 1);
+        }
+    }
+}
+
+// One wave per chunk.  Each iteration takes TPI = 64/K whole tokens, lane i <->
+// position chunk_begin + it*TPI*K + i, so the K slots of a token sit in one
+// iteration.  s_next[e] is the next free slot of expert e for this chunk.
+__global__ __launch_bounds__(kWave) void scatter_kernel(const uint16_t* __restrict__ compact,
+                                                        int64_t num_tokens, int64_t tokens_per_chunk,
+                                                        int E, int K, int ebits,
+                                                        const int32_t* __restrict__ chunk_base,
+                                                        const int64_t* __restrict__ offsets,
+                                                        int64_t* __restrict__ gate_index,
+                                                        int64_t* __restrict__ token_index,
+                                                        int64_t* __restrict__ reverse_index) {
+    extern __shared__ int32_t s_next[];
+    const int c = blockIdx.x;
+    const int lane = threadIdx.x;
+    for (int e = lane; e < E; e += kWave)
+        s_next[e] = (int32_t)offsets[e] + chunk_base[(int64_t)c * E + e];
+    __syncthreads();
+    const int tpi = kWave / K;
+    const int64_t t_begin = (int64_t)c * tokens_per_chunk;
+    int64_t t_end = t_begin + tokens_per_chunk;
+    if (t_end > num_tokens) t_end = num_tokens;
+    const int tok_in_iter = lane / K;
+    const int slot = lane - tok_in_iter * K;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (int64_t t0 = t_begin; t0 < t_end; t0 += tpi) {
+        const int64_t t = t0 + tok_in_iter;
+        const bool live = tok_in_iter < tpi && t < t_end;
+        const int64_t p = t * K + slot;
+        const uint32_t e = live ? compact[p] : (uint32_t)kBadExpert;
+        const bool counted = live && e != kBadExpert;
+        // lanes holding the same expert id
+        uint64_t same = __ballot(counted);
+        for (int b = 0; b < ebits; ++b) {
+            const uint64_t bal = __ballot((e >> b) & 1u);
+            same &= ((e >> b) & 1u) ? bal : ~bal;
+        }
+        const int before = __popcll(same & lt_mask);
+        const int count = __popcll(same);
+        int32_t base = 0;
+        if (counted) base = s_next[e];
+        __syncthreads();
+        if (counted && before == 0) s_next[e] = base + count;
+        __syncthreads();
+        const int64_t dst = (int64_t)base + before;
+        // rank of this slot among the token's K slots, ordered by (expert, slot)
+        int rank = 0;
+        for (int j = 0; j < K; ++j) {
+            const uint32_t oe = __shfl(e, tok_in_iter * K + j, kWave);
+            rank += (oe < e || (oe == e && j < slot)) ? 1 : 0;
+        }
+        if (counted) {
+            gate_index[dst] = p;
+            token_index[dst] = t;
+            reverse_index[t * K + rank] = dst;
+        }
+    }
+}
+
+int ceil_log2(int v) {
+    int b = 0;
+    while ((1 << b) < v) ++b;
+    return b;
+}
+
+int launch_sort(const uint16_t* compact, int32_t* chunk_hist, const RoutePlan& plan, int64_t T, int E,
+                int K, int64_t* lengths, int64_t* offsets, int64_t* gate_index, int64_t* token_index,
+                int64_t* reverse_index, hipStream_t stream) {
+    const int64_t total_pos = T * K;
+    hist_kernel<<<plan.num_chunks, kWave, E * sizeof(int32_t), stream>>>(
+        compact, total_pos, plan.tokens_per_chunk * K, E, chunk_hist);
+    int EW = 1;
+    while (EW < E) EW <<= 1;
+    scan_kernel<<<1, kScanThreads, kScanThreads * sizeof(int32_t), stream>>>(
+        chunk_hist, plan.num_chunks, E, EW, lengths, offsets);
+    scatter_kernel<<<plan.num_chunks, kWave, E * sizeof(int32_t), stream>>>(
+        compact, T, plan.tokens_per_chunk, E, K, ceil_log2(E), chunk_hist, offsets, gate_index,
+        token_index, reverse_index);
+    return check_launch("routing sort");
+}
+
+template <typename T, int LPT, int VPL>
+void launch_topk(const void* scores, int64_t T_, int E, int K, int renorm, int64_t* topk_idx,
+                 void* gates, uint16_t* compact, hipStream_t stream) {
+    constexpr int tokens_per_block = (256 / kWave) * (kWave / LPT);
+    const int64_t blocks = (T_ + tokens_per_block - 1) / tokens_per_block;
+    topk_kernel<T, LPT, VPL><<<(unsigned)blocks, 256, 0, stream>>>(
+        (const T*)scores, T_, E, K, renorm, topk_idx, (T*)gates, compact);
+}
+
+template <typename T>
+int dispatch_topk(const void* scores, int64_t T_, int E, int K, int renorm, int64_t* topk_idx,
+                  void* gates, uint16_t* compact, hipStream_t stream) {
+#define FMOE_TOPK(LPT, VPL) launch_topk<T, LPT, VPL>(scores, T_, E, K, renorm, topk_idx, gates, compact, stream)
+    if (E <= 8) FMOE_TOPK(8, 1);
+    else if (E <= 16) FMOE_TOPK(16, 1);
+    else if (E <= 32) FMOE_TOPK(32, 1);
+    else if (E <= 64) FMOE_TOPK(64, 1);
+    else if (E <= 128) FMOE_TOPK(64, 2);
+    else if (E <= 256) FMOE_TOPK(64, 4);
+    else if (E <= 512) FMOE_TOPK(64, 8);
+    else return fail(FMOE_ERR_UNSUPPORTED, "fmoe_route_topk: E=%d > 512", E);
+#undef FMOE_TOPK
+    return FMOE_OK;
+}
+
+int check_common(int64_t T, int E, int K, const void* workspace, size_t ws_bytes, const char* who) {
+    FMOE_REQUIRE(T >= 0 && E >= 1 && K >= 1, "%s: need T >= 0, E >= 1, K >= 1 (T=%lld E=%d K=%d)", who,
+                 (long long)T, E, K);
+    FMOE_REQUIRE(K <= 64, "%s: K=%d > 64 is not supported", who, K);
+    FMOE_REQUIRE(E <= 1024, "%s: E=%d > 1024 is not supported", who, E);
+    FMOE_REQUIRE(T * (int64_t)K < (int64_t)1 << 31, "%s: T*K must be below 2^31", who);
+    const RoutePlan plan = make_plan(T, E, K);
+    if (T > 0) {
+        FMOE_REQUIRE(workspace != nullptr, "%s: workspace is NULL", who);
+        if (ws_bytes < plan.total_bytes)
+            return fail(FMOE_ERR_WORKSPACE, "%s: workspace %zu B < required %zu B", who, ws_bytes,
+                        plan.total_bytes);
+    }
+    return FMOE_OK;
+}
+
+__global__ void empty_routing_kernel(int E, int64_t* lengths, int64_t* offsets) {
+    for (int e = threadIdx.x; e < E; e += blockDim.x) lengths[e] = 0;
+    for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = 0;
+}
+
+}  // namespace
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" size_t fmoe_route_workspace_bytes(int64_t T, int E, int K) {
+    if (T < 0 || E < 1 || K < 1) return 0;
+    return make_plan(T, E, K).total_bytes;
+}
+
+extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
+                               int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
+                               int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
+                               void* workspace, size_t workspace_bytes, fmoe_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (int rc = check_common(T, E, K, workspace, workspace_bytes, "fmoe_route_topk")) return rc;
+    FMOE_REQUIRE(K <= E, "fmoe_route_topk: K=%d > E=%d", K, E);
+    FMOE_REQUIRE(score_dtype == FMOE_F32 || score_dtype == FMOE_BF16,
+                 "fmoe_route_topk: scores must be fp32 or bf16");
+    FMOE_REQUIRE(lengths && offsets, "fmoe_route_topk: lengths/offsets are NULL");
+    if (T == 0) {
+        empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets);
+        return check_launch("fmoe_route_topk");
+    }
+    FMOE_REQUIRE(scores && topk_idx && gates && gate_index && token_index && reverse_index,
+                 "fmoe_route_topk: NULL tensor pointer");
+    const RoutePlan plan = make_plan(T, E, K);
+    uint16_t* compact = (uint16_t*)workspace;
+    int32_t* chunk_hist = (int32_t*)((char*)workspace + plan.compact_bytes);
+    int rc = score_dtype == FMOE_F32
+                 ? dispatch_topk<float>(scores, T, E, K, renorm, topk_idx, gates, compact, stream)
+                 : dispatch_topk<uint16_t>(scores, T, E, K, renorm, topk_idx, gates, compact, stream);
+    if (rc) return rc;
+    return launch_sort(compact, chunk_hist, plan, T, E, K, lengths, offsets, gate_index, token_index,
+                       reverse_index, stream);
+}
+
+extern "C" int fmoe_route_from_topk(const int64_t* topk_idx, int64_t T, int E, int K, int64_t* lengths,
+                                    int64_t* offsets, int64_t* gate_index, int64_t* token_index,
+                                    int64_t* reverse_index, int64_t* bad_count, void* workspace,
+                                    size_t workspace_bytes, fmoe_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    if (int rc = check_common(T, E, K, workspace, workspace_bytes, "fmoe_route_from_topk")) return rc;
+    FMOE_REQUIRE(lengths && offsets, "fmoe_route_from_topk: lengths/offsets are NULL");
+    if (bad_count) zero_i64_kernel<<<1, 1, 0, stream>>>(bad_count);
+    if (T == 0) {
+        empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets);
+        return check_launch("fmoe_route_from_topk");
+    }
+    FMOE_REQUIRE(topk_idx && gate_index && token_index && reverse_index,
+                 "fmoe_route_from_topk: NULL tensor pointer");
+    const RoutePlan plan = make_plan(T, E, K);
+    uint16_t* compact = (uint16_t*)workspace;
+    int32_t* chunk_hist = (int32_t*)((char*)workspace + plan.compact_bytes);
+    const int64_t n = T * K;
+    compact_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(topk_idx, n, E, compact, bad_count);
+    return launch_sort(compact, chunk_hist, plan, T, E, K, lengths, offsets, gate_index, token_index,
+                       reverse_index, stream);
+}

@@ -1,0 +1,298 @@
+"""Tensor-level wrappers over the C ABI: argument checks, output allocation,
+stride marshalling and the current-stream hand-off.  PyTorch is used for device
+memory and streams only; every computation below happens in libfastmoe_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import EPI_NONE, EPI_SILU, EPI_SWIGLU, FMOE_BF16, FMOE_E4M3, FMOE_F32, GemmDesc
+
+_DTYPE_CODE = {torch.float32: FMOE_F32, torch.bfloat16: FMOE_BF16}
+FP8_DTYPE = torch.float8_e4m3fn
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need_cuda(name: str, *tensors: Optional[torch.Tensor]) -> torch.device:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError(f"{name}: all tensors must live on the GPU (got a {t.device} tensor); "
+                             f"fast_moe_amd has no CPU path")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError(f"{name}: tensors on different devices ({dev} and {t.device})")
+    return dev
+
+
+def _forward_only(name: str, *tensors: Optional[torch.Tensor]) -> None:
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors):
+        raise RuntimeError(f"{name}: the HIP back-end is forward-only; call it under torch.no_grad() "
+                           f"or detach the inputs")
+
+
+def _i64(name: str, t: torch.Tensor) -> torch.Tensor:
+    if t.dtype != torch.int64:
+        raise ValueError(f"{name} must be int64, got {t.dtype}")
+    return t.contiguous()
+
+
+def _rows_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """Last dimension contiguous (the reference's switch_to_contiguous_if_needed)."""
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+# ------------------------------------------------------------------- routing
+def route_topk(scores: torch.Tensor, k: int, renorm: bool = True) -> Dict[str, torch.Tensor]:
+    """scores [T, E] (fp32 / bf16 gate probabilities) -> routing tensors, see fmoe_route_topk."""
+    dev = _need_cuda("route_topk", scores)
+    if scores.ndim != 2:
+        raise ValueError("route_topk: scores must be [T, E]")
+    if scores.dtype not in _DTYPE_CODE:
+        raise ValueError(f"route_topk: scores must be fp32 or bf16, got {scores.dtype}")
+    scores = scores.contiguous()
+    T, E = scores.shape
+    i64 = dict(dtype=torch.int64, device=dev)
+    out = {
+        "topk_idx": torch.empty((T, k), **i64),
+        "gates": torch.empty((T, k), dtype=scores.dtype, device=dev),
+        "lengths": torch.empty((E,), **i64),
+        "offsets": torch.empty((E + 1,), **i64),
+        "gate_index": torch.empty((T * k,), **i64),
+        "token_index": torch.empty((T * k,), **i64),
+        "reverse_index": torch.empty((T, k), **i64),
+    }
+    lib = _lib.load()
+    ws_bytes = lib.fmoe_route_workspace_bytes(T, E, k)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    rc = lib.fmoe_route_topk(
+        scores.data_ptr(), _DTYPE_CODE[scores.dtype], T, E, k, int(renorm),
+        out["topk_idx"].data_ptr(), out["gates"].data_ptr(), out["lengths"].data_ptr(),
+        out["offsets"].data_ptr(), out["gate_index"].data_ptr(), out["token_index"].data_ptr(),
+        out["reverse_index"].data_ptr(), ws.data_ptr(), ws_bytes, _stream(scores))
+    _lib.check(rc, "fmoe_route_topk")
+    return out
+
+
+def route_from_topk(topk_idx: torch.Tensor, num_experts: int) -> Dict[str, torch.Tensor]:
+    """topk_idx [T, K] int64 expert ids -> routing tensors, see fmoe_route_from_topk."""
+    dev = _need_cuda("route_from_topk", topk_idx)
+    if topk_idx.ndim != 2:
+        raise ValueError("route_from_topk: topk_idx must be [T, K]")
+    topk_idx = _i64("topk_idx", topk_idx)
+    T, k = topk_idx.shape
+    E = num_experts
+    i64 = dict(dtype=torch.int64, device=dev)
+    out = {
+        "lengths": torch.empty((E,), **i64),
+        "offsets": torch.empty((E + 1,), **i64),
+        "gate_index": torch.empty((T * k,), **i64),
+        "token_index": torch.empty((T * k,), **i64),
+        "reverse_index": torch.empty((T, k), **i64),
+        "bad_count": torch.empty((1,), **i64),
+    }
+    lib = _lib.load()
+    ws_bytes = lib.fmoe_route_workspace_bytes(T, E, k)
+    ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+    rc = lib.fmoe_route_from_topk(
+        topk_idx.data_ptr(), T, E, k, out["lengths"].data_ptr(), out["offsets"].data_ptr(),
+        out["gate_index"].data_ptr(), out["token_index"].data_ptr(), out["reverse_index"].data_ptr(),
+        out["bad_count"].data_ptr(), ws.data_ptr(), ws_bytes, _stream(topk_idx))
+    _lib.check(rc, "fmoe_route_from_topk")
+    return out
+
+
+# ---------------------------------------------------------------- fp8 quant
+def quant_rows_fp8(a: torch.Tensor, apply_silu: bool = False, reciprocal_scale: bool = False,
+                   out_like_input: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Row-wise (last dim) e4m3fn quantisation of ``a`` [..., rows, cols] read through its strides.
+
+    Returns ``(q, scale)``: q is float8_e4m3fn, contiguous in a's logical shape (or laid out
+    with a's own strides when ``out_like_input``), scale is fp32 with a's leading shape."""
+    dev = _need_cuda("quant_rows_fp8", a)
+    if a.dtype not in _DTYPE_CODE:
+        raise ValueError(f"quant_rows_fp8: input must be fp32 or bf16, got {a.dtype}")
+    if a.ndim < 1 or a.shape[-1] < 1:
+        raise ValueError("quant_rows_fp8: need at least one column")
+    shape = tuple(a.shape)
+    if a.ndim == 1:
+        a3 = a.view(1, 1, -1)
+    elif a.ndim == 2:
+        a3 = a.unsqueeze(0)
+    elif a.ndim == 3:
+        a3 = a
+    else:
+        a3 = a.reshape(-1, shape[-2], shape[-1])     # may copy for exotic >3-D strides
+    B, Rr, C = a3.shape
+    if out_like_input:
+        q3 = torch.empty_strided(a3.shape, a3.stride(), dtype=torch.uint8, device=dev)
+    else:
+        q3 = torch.empty(a3.shape, dtype=torch.uint8, device=dev)
+    scale = torch.empty((B, Rr), dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    rc = lib.fmoe_quant_rows_e4m3(
+        a3.data_ptr(), _DTYPE_CODE[a.dtype], B, Rr, C, a3.stride(0), a3.stride(1), a3.stride(2),
+        int(apply_silu), q3.data_ptr(), q3.stride(0), q3.stride(1), q3.stride(2), scale.data_ptr(),
+        int(reciprocal_scale), _stream(a))
+    _lib.check(rc, "fmoe_quant_rows_e4m3")
+    q = q3.view(FP8_DTYPE)
+    if a.ndim == 1:
+        q = q[0, 0]
+    elif a.ndim == 2:
+        q = q[0]
+    elif a.ndim > 3:
+        q = q.view(shape)
+    return q, scale.view(shape[:-1])
+
+
+# -------------------------------------------------------------- grouped GEMM
+def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, total_rows: int,
+                 row_index: Optional[torch.Tensor] = None, index_div: int = 1,
+                 bias: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None,
+                 bias2: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE, a_silu: bool = False,
+                 a_scale: Optional[torch.Tensor] = None, b_scale: Optional[torch.Tensor] = None,
+                 b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0) -> torch.Tensor:
+    """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
+    strides (bf16) or float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns bf16
+    [total_rows, N]."""
+    dev = _need_cuda("grouped_gemm", offsets, a, b, row_index, bias, b2, bias2, a_scale, b_scale, b2_scale)
+    fp8 = a.dtype == FP8_DTYPE
+    if not fp8 and a.dtype != torch.bfloat16:
+        raise NotImplementedError(
+            f"grouped_gemm: the HIP kernels take bf16 or float8_e4m3fn operands, got {a.dtype}")
+    if b.dtype != a.dtype or (b2 is not None and b2.dtype != a.dtype):
+        raise ValueError("grouped_gemm: A and B must share a dtype")
+    if b.ndim != 3:
+        raise ValueError("grouped_gemm: B must be [E, K, N]")
+    E, K, N = b.shape
+    if a.ndim not in (2, 3) or a.shape[-1] != K:
+        raise ValueError(f"grouped_gemm: A must be [rows, {K}] (or [rows, E, {K}]), got {tuple(a.shape)}")
+    if (a.ndim == 3) != (a_expert_stride != 0):
+        raise ValueError("grouped_gemm: a 3-D A needs a_expert_stride and vice versa")
+    if b2 is not None and (tuple(b2.shape) != (E, K, N) or b2.stride() != b.stride()):
+        raise ValueError("grouped_gemm: b2 must match b in shape and strides")
+    if offsets.numel() != E + 1:
+        raise ValueError(f"grouped_gemm: offsets must have E+1={E + 1} entries")
+    a = _rows_contiguous(a)
+    offsets = _i64("offsets", offsets)
+    if row_index is not None:
+        row_index = _i64("row_index", row_index).view(-1)
+        if row_index.numel() != total_rows:
+            raise ValueError("grouped_gemm: row_index must have total_rows entries")
+    out = torch.empty((total_rows, N), dtype=torch.bfloat16, device=dev)
+    if total_rows == 0:
+        return out
+
+    def bias_ok(t):
+        if t is None:
+            return None
+        if t.dtype != torch.bfloat16 or tuple(t.shape) != (E, N):
+            raise ValueError("grouped_gemm: bias must be bf16 [E, N]")
+        return _rows_contiguous(t)
+
+    bias, bias2 = bias_ok(bias), bias_ok(bias2)
+    if bias is not None and bias2 is not None and bias.stride(0) != bias2.stride(0):
+        bias2 = bias2.contiguous()
+        bias = bias.contiguous()
+    if fp8:
+        for name, s, n in (("a_scale", a_scale, a.shape[0] if a_expert_stride == 0 else None),
+                           ("b_scale", b_scale, E * N), ("b2_scale", b2_scale, E * N)):
+            if s is None:
+                if name == "b2_scale" and b2 is None:
+                    continue
+                raise ValueError(f"grouped_gemm: fp8 operands need {name}")
+            if s.dtype != torch.float32 or not s.is_contiguous() or (n is not None and s.numel() != n):
+                raise ValueError(f"grouped_gemm: {name} must be contiguous fp32 with one entry per row")
+
+    d = GemmDesc()
+    d.num_experts, d.n, d.k, d.index_div = E, N, K, index_div
+    d.total_rows = total_rows
+    d.a_rows = a.shape[0]
+    d.offsets = offsets.data_ptr()
+    d.row_index = _ptr(row_index)
+    d.a = a.data_ptr()
+    d.a_dtype = FMOE_E4M3 if fp8 else FMOE_BF16
+    d.a_silu = int(a_silu)
+    d.a_stride_row = a.stride(0)
+    d.a_stride_e = a_expert_stride
+    d.a_scale = _ptr(a_scale)
+    d.b = b.data_ptr()
+    d.b2 = _ptr(b2)
+    d.b_stride_e, d.b_stride_k, d.b_stride_n = b.stride()
+    d.b_scale = _ptr(b_scale)
+    d.b2_scale = _ptr(b2_scale)
+    d.bias = _ptr(bias)
+    d.bias2 = _ptr(bias2)
+    d.bias_stride_e = bias.stride(0) if bias is not None else (bias2.stride(0) if bias2 is not None else 0)
+    d.epilogue = epilogue
+    d.out_dtype = FMOE_BF16
+    d.out = out.data_ptr()
+    d.out_stride_row = out.stride(0)
+    rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
+    _lib.check(rc, "fmoe_grouped_gemm")
+    return out
+
+
+# ------------------------------------------------------------------ combine
+def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[torch.Tensor] = None,
+            gates_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Weighted merge, see fmoe_combine.  value [T*K, D]; reverse_index [T, K]."""
+    dev = _need_cuda("combine", value, reverse_index, gates, gates_index)
+    if value.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"combine: value must be fp32 or bf16, got {value.dtype}")
+    T, K = reverse_index.shape
+    D = value.shape[1]
+    value = _rows_contiguous(value)
+    reverse_index = _i64("reverse_index", reverse_index)
+    out_dtype = value.dtype
+    g_code, g_cols, g_sr, g_sc = FMOE_F32, 1, 1, 1
+    if gates is not None:
+        if gates.dtype not in _DTYPE_CODE:
+            raise NotImplementedError(f"combine: gates must be fp32 or bf16, got {gates.dtype}")
+        if gates.numel() != T * K:
+            raise ValueError(f"combine: gates has {gates.numel()} entries, expected {T * K}")
+        if gates.ndim == 1:
+            gates = gates.view(-1, 1)
+        if gates.ndim != 2:
+            gates = gates.contiguous().view(-1, 1)
+        out_dtype = torch.promote_types(value.dtype, gates.dtype)
+        g_code, g_cols, g_sr, g_sc = _DTYPE_CODE[gates.dtype], gates.shape[1], gates.stride(0), gates.stride(1)
+        if gates_index is not None:
+            gates_index = _i64("gates_index", gates_index).view(-1)
+            if gates_index.numel() != T * K:
+                raise ValueError("combine: gates_index must have T*K entries")
+    else:
+        gates_index = None
+    out = torch.empty((T, D), dtype=out_dtype, device=dev)
+    rc = _lib.load().fmoe_combine(
+        value.data_ptr(), _DTYPE_CODE[value.dtype], T, K, D, value.stride(0), reverse_index.data_ptr(),
+        _ptr(gates), g_code, g_cols, g_sr, g_sc, _ptr(gates_index), out.data_ptr(), _DTYPE_CODE[out_dtype],
+        _stream(value))
+    _lib.check(rc, "fmoe_combine")
+    return out
+
+
+def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """``silu(a) * b`` element-wise (bf16, contiguous, same shape)."""
+    _need_cuda("silu_mul", a, b)
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.shape != b.shape:
+        raise ValueError("silu_mul: two bf16 tensors of one shape expected")
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty_like(a)
+    rc = _lib.load().fmoe_silu_mul(a.data_ptr(), b.data_ptr(), out.data_ptr(), FMOE_BF16, a.numel(), _stream(a))
+    _lib.check(rc, "fmoe_silu_mul")
+    return out

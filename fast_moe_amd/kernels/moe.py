@@ -1,0 +1,193 @@
+"""bf16 operator API of the MoE forward -- the drop-in boundary.
+
+Function names, positional order, keyword names and argument meaning are those
+of /root/reference/kernels/moe.py:39-292.  Differences, all on purpose:
+
+* ``kernel`` defaults to ``KernelType.HIP`` (the reference defaults to its
+  PyTorch path, which this package does not contain); ``KernelType.TRITON`` is
+  accepted and runs the same HIP kernels; any other value raises.
+* forward only: inputs that require grad raise unless grad mode is off.
+* ``max_seq_len`` is accepted and ignored: tile scheduling reads ``offsets`` on
+  the device, so no host synchronisation is needed to obtain it.
+* operands must be bf16 CUDA tensors (fp32 for ``mul_merge_k_add``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from .hip import ops
+from .hip._lib import EPI_NONE, EPI_SWIGLU
+from .utils import KernelType, require_hip_kernel
+
+
+@dataclass
+class IndexSelectJaggedBmmOption:
+    """kernels/triton/triton_moe.py:36-43: backward-tuning knobs, accepted and unused."""
+    d_jagged_use_grouped_gemm: bool = True
+    d_jagged_use_wrap_specialization: bool = True
+    d_jagged_gemm_out_type: torch.dtype = torch.float32
+    d_weight_optimization: bool = True
+    d_weight_split_k_kernel: bool = True
+    d_weight_split_k_kernel_tma: bool = False
+
+
+@dataclass
+class SiluJaggedBmmCombineOption:
+    """kernels/triton/triton_moe.py:3562-3567: accepted and unused (backward only)."""
+    activation_checkpointing: bool = False
+    d_weight_optimization: bool = True
+    d_weight_split_k_kernel: bool = True
+    d_weight_split_k_kernel_tma: bool = False
+
+
+def _check_gather_args(name, index, jagged, weight):
+    assert index.ndim == 2 and index.shape[0] == jagged.shape[0], (
+        f"{name}: index must be [L, A] with L = jagged.shape[0]")
+    assert weight.ndim == 3, f"{name}: weight must be [E, K, N]"
+
+
+def index_select_jagged_bmm(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    index: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    kernel: KernelType = KernelType.HIP,
+    triton_option: Optional[IndexSelectJaggedBmmOption] = None,
+) -> torch.Tensor:
+    """kernels/moe.py:39-68.  ``out[off_e:off_e+1] = jagged[index[...] // A] @ weight[e] + bias[e]``."""
+    require_hip_kernel(kernel, "index_select_jagged_bmm")
+    _check_gather_args("index_select_jagged_bmm", index, jagged, weight)
+    ops._forward_only("index_select_jagged_bmm", jagged, weight, bias)
+    return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
+                            index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
+
+
+def mul_merge_k_add(
+    index: torch.Tensor,
+    reverse_index: torch.Tensor,
+    value: torch.Tensor,
+    stable_sorting: bool = False,
+    weight: Optional[torch.Tensor] = None,
+    weight_index: Optional[torch.Tensor] = None,
+    kernel: KernelType = KernelType.HIP,
+    triton_cc_version: str = "",
+) -> torch.Tensor:
+    """kernels/moe.py:71-115.  ``out[n] = sum of value[r] * weight_flat[weight_index[r]]`` over the
+    K rows r = reverse_index[n, :], added in ascending r."""
+    require_hip_kernel(kernel, "mul_merge_k_add")
+    N = index.shape[0]
+    L, K = reverse_index.shape
+    assert index.ndim == 1 and reverse_index.ndim == 2
+    assert N == L * K and N == value.shape[0]
+    if weight is not None:
+        assert weight_index is not None
+        assert weight.numel() == weight_index.numel() == value.shape[0], (
+            f"{weight.shape=}, {weight_index.shape=}, {value.shape=}")
+    ops._forward_only("mul_merge_k_add", value, weight)
+    return ops.combine(value, reverse_index, weight, weight_index)
+
+
+def index_select_jagged_bmm_3D(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    index: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor,
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/moe.py:118-153.  jagged [L, E, D_in]: expert e reads slice ``[:, e, :]``."""
+    require_hip_kernel(kernel, "index_select_jagged_bmm_3D")
+    assert index.ndim == 2 and index.shape[0] == jagged.shape[0]
+    assert jagged.ndim == 3 and jagged.shape[1] == weight.shape[0]
+    ops._forward_only("index_select_jagged_bmm_3D", jagged, weight, bias)
+    jagged = ops._rows_contiguous(jagged)
+    return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
+                            index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE,
+                            a_expert_stride=jagged.stride(1))
+
+
+def index_select_jagged_bmm_swiglu(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    index: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    weight_p: torch.Tensor,
+    bias_p: Optional[torch.Tensor],
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/moe.py:156-189.  ``silu(x W + b) * (x Wp + bp)`` in one kernel."""
+    require_hip_kernel(kernel, "index_select_jagged_bmm_swiglu")
+    _check_gather_args("index_select_jagged_bmm_swiglu", index, jagged, weight)
+    assert weight.shape == weight_p.shape
+    ops._forward_only("index_select_jagged_bmm_swiglu", jagged, weight, bias, weight_p, bias_p)
+    if weight_p.stride() != weight.stride():
+        weight_p = weight_p.contiguous()
+        weight = weight.contiguous()
+    return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
+                            index_div=index.shape[-1], bias=bias, b2=weight_p, bias2=bias_p,
+                            epilogue=EPI_SWIGLU)
+
+
+def index_select_jagged_gating_bmm(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    index: torch.Tensor,
+    jagged_a: torch.Tensor,
+    jagged_b: torch.Tensor,
+    weight_a: torch.Tensor,
+    bias_a: Optional[torch.Tensor],
+    weight_b: torch.Tensor,
+    bias_b: Optional[torch.Tensor],
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/moe.py:192-233.  ``silu(A Wa + ba) * (B Wb + bb)``; one fused kernel when A is B,
+    otherwise two GEMMs and an element-wise kernel."""
+    require_hip_kernel(kernel, "index_select_jagged_gating_bmm")
+    assert (index.ndim == 2 and index.shape[0] == jagged_a.shape[0] == jagged_b.shape[0]
+            and jagged_a.shape == jagged_b.shape and weight_a.shape == weight_b.shape)
+    if jagged_a is jagged_b:
+        return index_select_jagged_bmm_swiglu(max_seq_len, offsets, index, jagged_a, weight_a, bias_a,
+                                              weight_b, bias_b, kernel)
+    ops._forward_only("index_select_jagged_gating_bmm", jagged_a, jagged_b, weight_a, weight_b, bias_a, bias_b)
+    alpha = ops.grouped_gemm(offsets, jagged_a, weight_a, total_rows=index.numel(), row_index=index,
+                             index_div=index.shape[-1], bias=bias_a)
+    beta = ops.grouped_gemm(offsets, jagged_b, weight_b, total_rows=index.numel(), row_index=index,
+                            index_div=index.shape[-1], bias=bias_b)
+    return ops.silu_mul(alpha, beta)
+
+
+def silu_jagged_bmm_combine(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    index: torch.Tensor,
+    reverse_index: torch.Tensor,
+    gating_scores: Optional[torch.Tensor] = None,
+    gates_index: Optional[torch.Tensor] = None,
+    has_silu: bool = True,
+    kernel: KernelType = KernelType.HIP,
+    triton_option: Optional[SiluJaggedBmmCombineOption] = None,
+) -> torch.Tensor:
+    """kernels/moe.py:236-292.  ``silu(jagged) @ weight[e] + bias[e]`` on expert-sorted rows, then
+    the weighted merge of the K rows of each token."""
+    if kernel == KernelType.TRITON_CC:
+        raise NotImplementedError("TRITON_CC is not supported for silu_jagged_bmm_combine")
+    require_hip_kernel(kernel, "silu_jagged_bmm_combine")
+    N = index.shape[0]
+    L, K = reverse_index.shape
+    assert index.ndim == 1 and reverse_index.ndim == 2
+    assert N == L * K and N == jagged.shape[0], f"{N=}, {L=}, {K=}, {jagged.shape=}"
+    ops._forward_only("silu_jagged_bmm_combine", jagged, weight, bias, gating_scores)
+    bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=N, bias=bias, epilogue=EPI_NONE,
+                               a_silu=has_silu)
+    return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)

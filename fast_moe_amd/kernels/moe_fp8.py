@@ -1,0 +1,135 @@
+"""FP8 (OCP e4m3fn, row-wise power-of-two scales) operator API.
+
+Names, argument order and meaning follow /root/reference/kernels/moe_fp8.py:31-248.
+``kernel`` defaults to ``KernelType.HIP``; ``TRITON`` selects the same kernels.
+Where the reference's two back-ends disagree on a weight layout
+(kernels/triton/triton_moe_fp8.py:1393 reads [E, D_out, D_in] while the PyTorch
+branch of the same operator reads [E, D_in, D_out]) the layout of the PyTorch
+branch -- the one every bf16 operator uses -- is taken: weights are [E, D_in, D_out]
+tensors of any strides, except ``silu_jagged_bmm_fp8`` which keeps the
+[E, D_out, D_in] layout of its only runnable reference implementation.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .hip import ops
+from .hip._lib import EPI_NONE
+from .utils import KernelType, require_hip_kernel
+
+
+def rowwise_quant_fp8(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """kernels/pytorch/quant_fp8.py:27-34: ``(a_fp8, a_scale)`` with the MULTIPLIER scale."""
+    return ops.quant_rows_fp8(a)
+
+
+def transpose_rowwise_quant_fp8(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """kernels/pytorch/quant_fp8.py:37-40: quantise ``a.transpose(-2, -1)`` row-wise (no copy of a)."""
+    return ops.quant_rows_fp8(a.transpose(-2, -1))
+
+
+def quantize_expert_weights(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Weight [E, K, N] (any strides) -> (fp8 [E, K, N] view of [E, N, K] storage, scale [E, N]):
+    one scale per (expert, output row), K-contiguous bytes ready for the fp8 GEMM.  This is the
+    quantisation kernels/pytorch/moe_fp8.py:111 redoes on every call; do it once per weight update."""
+    q, s = ops.quant_rows_fp8(weight.permute(0, 2, 1))     # [E, N, K] contiguous
+    return q.permute(0, 2, 1), s
+
+
+def silu_jagged_fp8(
+    seq_offsets: torch.Tensor,
+    Jagged: torch.Tensor,
+    max_seq_len: int,
+    K: int,
+    Silu_Jagged: torch.Tensor,
+    Silu_Jagged_fp8: torch.Tensor,
+    Silu_Jagged_Scale: torch.Tensor,
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/moe_fp8.py:31-74: ``silu(Jagged)`` quantised per row; returns the fp8 tensor.  Like
+    the reference's PyTorch path, the three buffer arguments are not written."""
+    require_hip_kernel(kernel, "silu_jagged_fp8")
+    q, _ = ops.quant_rows_fp8(Jagged, apply_silu=True)
+    return q
+
+
+def bmm_weight_rowwise_quant_fp8(weight: torch.Tensor, kernel: KernelType = KernelType.HIP) -> torch.Tensor:
+    """kernels/moe_fp8.py:77-95: weight [E, D_in, D_out], one scale per (expert, output column)
+    from the amax over D_in; returns the fp8 weight in the same [E, D_in, D_out] layout."""
+    require_hip_kernel(kernel, "bmm_weight_rowwise_quant_fp8")
+    q, _ = ops.quant_rows_fp8(weight.permute(0, 2, 1), out_like_input=True)
+    return q.permute(0, 2, 1)
+
+
+def silu_jagged_bmm_fp8(
+    seq_offsets: torch.Tensor,
+    max_seq_len: int,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor,
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/moe_fp8.py:98-124 with weight [E, D_out, D_in] (kernels/pytorch/moe_fp8.py:46-75):
+    ``silu(jagged)`` row-quantised, weight row-quantised, fp8 GEMM + bias."""
+    require_hip_kernel(kernel, "silu_jagged_bmm_fp8")
+    ops._forward_only("silu_jagged_bmm_fp8", jagged, weight, bias)
+    qa, sa = ops.quant_rows_fp8(jagged, apply_silu=True)
+    qw, sw = ops.quant_rows_fp8(weight)                      # rows of [E, D_out, D_in]
+    return ops.grouped_gemm(seq_offsets, qa, qw.permute(0, 2, 1), total_rows=jagged.shape[0], bias=bias,
+                            a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
+
+
+def silu_jagged_bmm_combine_fp8(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    index: torch.Tensor,
+    reverse_index: torch.Tensor,
+    gating_scores: Optional[torch.Tensor] = None,
+    gates_index: Optional[torch.Tensor] = None,
+    activation_checkpointing: bool = False,
+    has_silu: bool = True,
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/moe_fp8.py:127-182: (SiLU +) row-quant of the hidden, weight row-quant, fp8 grouped
+    GEMM + bias, weighted merge.  weight is [E, D_in, D_out]."""
+    require_hip_kernel(kernel, "silu_jagged_bmm_combine_fp8")
+    L, K = reverse_index.shape
+    assert index.shape[0] == L * K == jagged.shape[0]
+    ops._forward_only("silu_jagged_bmm_combine_fp8", jagged, weight, bias, gating_scores)
+    qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
+    qw, sw = quantize_expert_weights(weight)
+    bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias, a_scale=sa,
+                               b_scale=sw, epilogue=EPI_NONE)
+    return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
+
+
+def index_select_jagged_bmm(
+    max_seq_len: int,
+    offsets: torch.Tensor,
+    index: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    kernel: KernelType = KernelType.HIP,
+    fp8: bool = False,
+) -> torch.Tensor:
+    """kernels/moe_fp8.py:185-248.  fp8=True: tokens quantised per row BEFORE the gather, weight
+    per output row, fp8 MFMA GEMM, ``acc / (s_a x s_w)`` cast to bf16, plus bias
+    (kernels/pytorch/moe_fp8.py:98-139).  fp8=False: the bf16 operator."""
+    require_hip_kernel(kernel, "index_select_jagged_bmm")
+    assert index.ndim == 2 and index.shape[0] == jagged.shape[0]
+    ops._forward_only("index_select_jagged_bmm", jagged, weight, bias)
+    if not fp8:
+        return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
+                                index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
+    assert jagged.dtype == weight.dtype and (bias is None or jagged.dtype == bias.dtype)
+    qa, sa = ops.quant_rows_fp8(jagged)
+    qw, sw = quantize_expert_weights(weight)
+    return ops.grouped_gemm(offsets, qa, qw, total_rows=index.numel(), row_index=index,
+                            index_div=index.shape[-1], bias=bias, a_scale=sa, b_scale=sw,
+                            epilogue=EPI_NONE)

@@ -1,0 +1,38 @@
+"""Kernel selector and small helpers of the operator API.
+
+Mirrors /root/reference/kernels/utils.py:13-33.  ``KernelType`` keeps the
+reference's members so that existing call sites type-check, and gains ``HIP``:
+the hand-written gfx950 back-end, which is the only back-end this package ships.
+``TRITON`` (the reference's GPU back-end) is served by the same HIP kernels;
+``PYTORCH`` and ``TRITON_CC`` raise, because no PyTorch or CPU fallback exists
+in this package.
+"""
+from __future__ import annotations
+
+from enum import Enum, unique
+
+import torch
+
+
+@unique
+class KernelType(Enum):
+    TRITON = "TRITON"
+    PYTORCH = "PYTORCH"
+    TRITON_CC = "TRITON_CC"
+    HIP = "HIP"
+
+
+def require_hip_kernel(kernel: "KernelType", op: str) -> None:
+    """Every operator funnels its ``kernel`` argument through this check."""
+    if kernel in (KernelType.HIP, KernelType.TRITON):
+        return
+    raise NotImplementedError(
+        f"{op}: kernel={kernel} is not available; fast_moe_amd ships only the MI355X HIP "
+        f"back-end (KernelType.HIP, also selected by KernelType.TRITON) and has no PyTorch/CPU path")
+
+
+def to_fp32_if_pytorch_kernel(x: torch.Tensor, kernel: KernelType = KernelType.PYTORCH) -> torch.Tensor:
+    """kernels/utils.py:28-33 (test helper kept for signature compatibility)."""
+    if kernel == KernelType.PYTORCH:
+        return x.to(torch.float32)
+    return x

@@ -1,0 +1,97 @@
+"""``FastMoELayer``: the MoE layer of /root/reference/modules/fast_moe_module.py:45-225
+on the MI355X HIP back-end.
+
+Constructor arguments, parameter names / shapes / dtypes (so state_dicts
+interchange) and ``forward(x, num_experts_per_tok)`` are the reference's.  The
+gate (Linear + softmax) stays a torch call; everything after it -- top-k, gate
+renormalisation, routing tensors, both expert GEMMs, SiLU and the weighted
+merge -- runs in libfastmoe_hip.so with no host synchronisation (the reference
+syncs once for ``max_seq_len``, fast_moe_module.py:135).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.autograd.profiler import record_function
+
+from ..kernels.hip import ops
+from ..kernels.hip._lib import EPI_NONE, EPI_SILU
+from ..kernels.utils import KernelType, require_hip_kernel
+
+
+def _create_fused_mlp_weights(num_mlps: int, in_dim: int, out_dim: int) -> torch.Tensor:
+    """utils/utils.py:38-42: one xavier-uniform [in_dim, out_dim] matrix per expert."""
+    t = torch.empty(size=(num_mlps, in_dim, out_dim))
+    for i in range(num_mlps):
+        torch.nn.init.xavier_uniform_(t[i])
+    return t
+
+
+class GatingNetwork(nn.Module):
+    """fast_moe_module.py:21-27."""
+
+    def __init__(self, input_dim: int, num_experts: int) -> None:
+        super().__init__()
+        self.gate = nn.Linear(input_dim, num_experts)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.softmax(self.gate(x), dim=2)
+
+
+class FastMoELayer(nn.Module):
+    def __init__(
+        self,
+        input_dim: int,
+        hidden_dim: int,
+        output_dim: int,
+        num_experts: int,
+        kernel: KernelType = KernelType.HIP,
+        dtype: torch.dtype = torch.bfloat16,
+    ) -> None:
+        super().__init__()
+        self.input_dim: int = input_dim
+        self.hidden_dim: int = hidden_dim
+        self.output_dim: int = output_dim
+        self.num_experts: int = num_experts
+        self.kernel: KernelType = kernel
+        self.dtype: torch.dtype = dtype
+
+        self.gate = GatingNetwork(input_dim, num_experts)
+        self._experts_hidden_w = nn.Parameter(
+            _create_fused_mlp_weights(num_experts, hidden_dim, input_dim).to(dtype=dtype))
+        self._experts_hidden_bias = nn.Parameter(torch.zeros([num_experts, hidden_dim], dtype=dtype))
+        self._experts_w = nn.Parameter(
+            _create_fused_mlp_weights(num_experts, output_dim, hidden_dim).to(dtype=dtype))
+        self._experts_bias = nn.Parameter(torch.zeros([num_experts, output_dim], dtype=dtype))
+
+    def route(self, x: torch.Tensor, num_experts_per_tok: int) -> Dict[str, torch.Tensor]:
+        """fast_moe_module.py:93-144 in one library call on the gate probabilities."""
+        scores = self.gate(x).reshape(-1, self.num_experts)
+        return ops.route_topk(scores, num_experts_per_tok, renorm=True)
+
+    def forward(self, x: torch.Tensor, num_experts_per_tok: int) -> torch.Tensor:
+        require_hip_kernel(self.kernel, "FastMoELayer.forward")
+        if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
+            raise RuntimeError("FastMoELayer: the HIP back-end is forward-only; call it under "
+                               "torch.no_grad() / torch.inference_mode()")
+        if x.dtype != torch.bfloat16:
+            raise NotImplementedError(f"FastMoELayer: the HIP kernels take bf16 activations, got {x.dtype}")
+        original_shape = x.shape
+        k = num_experts_per_tok
+        r = self.route(x, k)
+        with record_function("## expert_forward##"):
+            x_flat = x.reshape(-1, self.input_dim)
+            # GEMM1 with SiLU in the epilogue: the hidden is rounded to bf16 before and after the
+            # activation, exactly as the two-operator form of fast_moe_module.py:162-184 rounds it
+            hidden = ops.grouped_gemm(
+                r["offsets"], x_flat, self._experts_hidden_w.permute(0, 2, 1).to(x.dtype),
+                total_rows=x_flat.shape[0] * k, row_index=r["gate_index"], index_div=k,
+                bias=self._experts_hidden_bias.to(x.dtype), epilogue=EPI_SILU)
+            out_rows = ops.grouped_gemm(
+                r["offsets"], hidden, self._experts_w.permute(0, 2, 1).to(x.dtype),
+                total_rows=hidden.shape[0], bias=self._experts_bias.to(x.dtype), epilogue=EPI_NONE)
+            y = ops.combine(out_rows, r["reverse_index"], r["gates"], r["gate_index"])
+        return y.view(original_shape[0], original_shape[1], self.output_dim)

@@ -1,0 +1,221 @@
+/*
+ * fast_moe_amd -- C ABI of libfastmoe_hip.so: the MoE-forward hot path of
+ * meta-recsys/fast_moe as hand-written gfx950 (MI355X) HIP kernels.
+ *
+ * Conventions shared by every entry point
+ *   - plain pointers and sizes only; every pointer is a DEVICE pointer unless
+ *     stated otherwise; the caller owns all memory, the library allocates none,
+ *     keeps no pointer past the call and holds no global state;
+ *   - all work is enqueued on `stream` (a hipStream_t passed as void*) and the
+ *     call returns without synchronising the host;
+ *   - return value 0 = success; non-zero = error, message from fmoe_last_error()
+ *     (thread local).  Nothing is launched when an argument check fails;
+ *   - index tensors are int64 (what torch.sort / cumsum hand the reference),
+ *     row addressing is 64-bit inside.
+ *
+ * Reference citations are relative to the root of meta-recsys/fast_moe.
+ */
+#ifndef FAST_MOE_AMD_H
+#define FAST_MOE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* fmoe_stream_t; /* hipStream_t */
+
+enum fmoe_dtype {
+    FMOE_F32 = 0,
+    FMOE_BF16 = 1,
+    FMOE_E4M3 = 2 /* OCP float8 e4m3fn bytes + fp32 row scales */
+};
+
+enum fmoe_epilogue {
+    FMOE_EPI_NONE = 0,  /* out = acc + bias                                  */
+    FMOE_EPI_SILU = 1,  /* out = silu(round(acc + bias))                     */
+    FMOE_EPI_SWIGLU = 2 /* out = silu(round(acc + bias)) * round(acc2 + bias2) */
+};
+
+enum fmoe_status {
+    FMOE_OK = 0,
+    FMOE_ERR_ARGUMENT = 1,    /* bad shape / dtype / null pointer / alignment   */
+    FMOE_ERR_UNSUPPORTED = 2, /* valid request this build has no kernel for     */
+    FMOE_ERR_WORKSPACE = 3,   /* workspace too small                            */
+    FMOE_ERR_LAUNCH = 4       /* hipGetLastError() after a launch               */
+};
+
+/* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
+int fmoe_version(void);
+
+/* Message of the last non-zero return on this thread ("" if none). */
+const char* fmoe_last_error(void);
+
+/* ------------------------------------------------------------------ routing */
+
+/* Bytes of scratch fmoe_route_topk / fmoe_route_from_topk need for (T, E, K). */
+size_t fmoe_route_workspace_bytes(int64_t T, int E, int K);
+
+/*
+ * Top-k expert selection, L1 gate renormalisation and the jagged routing
+ * tensors, from gate probabilities.
+ * Replaces FastMoELayer._select_top_k_experts + _compute_routing_metadata
+ * (modules/fast_moe_module.py:93-144) including the third-party
+ * torch.ops.fbgemm.asynchronous_complete_cumsum call at :131.
+ *
+ *   scores        [T, E] row-major, FMOE_F32 or FMOE_BF16 (softmax output)
+ *   renorm        1: gates = v / max(sum|v|, 1e-12) in the scores' dtype
+ *                 (F.normalize, :103); 0: gates = selected scores
+ * outputs
+ *   topk_idx      [T, K] int64  selected experts; slot order = descending score,
+ *                               equal scores -> lower expert id first
+ *   gates         [T, K] scores' dtype
+ *   lengths       [E]    int64  rows per expert
+ *   offsets       [E+1]  int64  exclusive prefix sum of lengths
+ *   gate_index    [T*K]  int64  stable argsort of topk_idx.view(-1)      (:122)
+ *   token_index   [T*K]  int64  gate_index / K                           (:124)
+ *   reverse_index [T, K] int64  stable argsort of token_index            (:132)
+ * Limits: 1 <= K <= E <= 512, K <= 64.
+ */
+int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
+                    int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
+                    int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
+                    void* workspace, size_t workspace_bytes, fmoe_stream_t stream);
+
+/*
+ * The same routing tensors for a caller that already holds the selected expert
+ * ids (the generator of kernels/tests/moe_test.py:191-197,241: topk -> stable
+ * sort -> scatter_add -> complete cumsum).  topk_idx values must lie in [0, E);
+ * out-of-range ids are counted into no expert and reported through
+ * `bad_count` (device int64, may be NULL).  Limits: E <= 65536, K <= 64.
+ */
+int fmoe_route_from_topk(const int64_t* topk_idx, int64_t T, int E, int K,
+                         int64_t* lengths, int64_t* offsets, int64_t* gate_index,
+                         int64_t* token_index, int64_t* reverse_index, int64_t* bad_count,
+                         void* workspace, size_t workspace_bytes, fmoe_stream_t stream);
+
+/* ---------------------------------------------------------- FP8 quantisation */
+
+/*
+ * Row-wise OCP e4m3fn quantisation with a power-of-two multiplier scale
+ * 2^floor(log2(448/amax)) per row.
+ * Replaces pytorch_rowwise_quant_fp8 / pytorch_transpose_rowwise_quant_fp8
+ * (kernels/pytorch/quant_fp8.py:13-40), pytorch_silu_jagged_fp8 and
+ * pytorch_bmm_weight_rowwise_quant_fp8 (kernels/pytorch/moe_fp8.py:17-43),
+ * i.e. triton_rowwise_quant_fp8 & co (kernels/triton/triton_quant_fp8.py:130-302).
+ *
+ *   a      logical [batch, rows, cols] read through element strides a_stride_*;
+ *          the amax runs over `cols`.  FMOE_BF16 or FMOE_F32.
+ *   q      e4m3fn bytes written through element strides q_stride_*
+ *   scale  [batch, rows] fp32, contiguous: the multiplier, or its reciprocal
+ *          when store_reciprocal != 0 (the convention of
+ *          kernels/triton/triton_quant_fp8.py:273-277)
+ *   apply_silu  quantise silu(a) (rounded to a's dtype first) instead of a
+ */
+int fmoe_quant_rows_e4m3(const void* a, int a_dtype, int64_t batch, int64_t rows, int64_t cols,
+                         int64_t a_stride_b, int64_t a_stride_r, int64_t a_stride_c,
+                         int apply_silu, uint8_t* q, int64_t q_stride_b, int64_t q_stride_r,
+                         int64_t q_stride_c, float* scale, int store_reciprocal,
+                         fmoe_stream_t stream);
+
+/* -------------------------------------------------------------- grouped GEMM */
+
+/*
+ * One jagged ("grouped") GEMM over expert segments:
+ *   for e in [0, E), r in [offsets[e], offsets[e+1]):
+ *     src      = row_index ? row_index[r] / index_div : r
+ *     acc [n]  = sum_k A [src, k] * B [e, k, n]
+ *     acc2[n]  = sum_k A [src, k] * B2[e, k, n]              (SWIGLU only)
+ *     out[r,n] = epilogue(acc (+bias[e,n]), acc2 (+bias2[e,n]))
+ * With FMOE_E4M3 operands acc is divided by a_scale[src] * b_scale[e, n]
+ * (multiplier scales) before the bias, as kernels/pytorch/moe_fp8.py:127-137.
+ *
+ * Replaces, by choice of fields:
+ *   index_select_jagged_bmm          kernels/moe.py:39-68     (row_index, EPI_NONE)
+ *   index_select_jagged_bmm_swiglu   kernels/moe.py:156-189   (row_index, EPI_SWIGLU)
+ *   index_select_jagged_bmm_3D       kernels/moe.py:118-153   (a_stride_e != 0)
+ *   the GEMM half of silu_jagged_bmm_combine kernels/moe.py:236-292
+ *                                    (row_index NULL, a_silu = has_silu)
+ *   index_select_jagged_bmm(fp8=True) kernels/moe_fp8.py:185-248 (FMOE_E4M3)
+ *   the GEMM of silu_jagged_bmm_combine_fp8 kernels/moe_fp8.py:127-182
+ * i.e. the Triton kernels kernels/triton/triton_moe.py:184-282, 2526-2671,
+ * 3167-3347, kernels/triton/triton_moe_fp8.py:672-884 and
+ * kernels/triton/triton_gemm_fp8.py:55-204.
+ *
+ * All strides are in elements.  B is addressed as B[e*b_stride_e + k*b_stride_k
+ * + n*b_stride_n], so both [E,K,N]-contiguous weights and [E,K,N] views of
+ * [E,N,K] storage are consumed in place.  No host synchronisation: tile
+ * scheduling reads `offsets` on the device; max_seq_len is not needed.
+ */
+typedef struct fmoe_gemm_desc {
+    int32_t num_experts;    /* E                                                  */
+    int32_t n;              /* output columns (per B matrix)                      */
+    int32_t k;              /* contraction length                                 */
+    int32_t index_div;      /* divisor applied to row_index values (>= 1)         */
+    int64_t total_rows;     /* rows of `out` (= offsets[E]; host-known upper bound) */
+    int64_t a_rows;         /* rows of A (bound for gathered sources)             */
+    const int64_t* offsets; /* [E+1]                                              */
+    const int64_t* row_index; /* [total_rows] or NULL                             */
+
+    const void* a;          /* [a_rows, k] (or [a_rows, E, k] with a_stride_e)    */
+    int32_t a_dtype;        /* FMOE_BF16 | FMOE_E4M3                              */
+    int32_t a_silu;         /* apply SiLU to A elements on load (bf16 only)       */
+    int64_t a_stride_row;
+    int64_t a_stride_e;     /* 0, or per-expert offset for the 3D variant         */
+    const float* a_scale;   /* [a_rows] multiplier scales (FMOE_E4M3)             */
+
+    const void* b;          /* same dtype as A                                    */
+    const void* b2;         /* second weight (SWIGLU) or NULL                     */
+    int64_t b_stride_e, b_stride_k, b_stride_n;
+    const float* b_scale;   /* [E, n] multiplier scales (FMOE_E4M3)               */
+    const float* b2_scale;
+
+    const void* bias;       /* [E, n] in out_dtype, or NULL                       */
+    const void* bias2;
+    int64_t bias_stride_e;
+
+    int32_t epilogue;       /* enum fmoe_epilogue                                 */
+    int32_t out_dtype;      /* FMOE_BF16                                          */
+    void* out;              /* [total_rows, n]                                    */
+    int64_t out_stride_row;
+} fmoe_gemm_desc;
+
+int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);
+
+/* ------------------------------------------------------------------ combine */
+
+/*
+ * Weighted, deterministic merge of the K expert rows of each token:
+ *   out[t, :] = sum_{j<K} round(value[reverse_index[t,j], :] * w(reverse_index[t,j]))
+ * accumulated in fp32 in ascending j (= ascending source row, the order of the
+ * reference's CPU index_add), where w(r) = gates_flat[gates_index[r]]
+ * (or gates_flat[r] if gates_index is NULL, or 1 if gates is NULL) and the
+ * product is rounded to the promoted dtype of (value, gates) before the add.
+ * Replaces pytorch_mul_merge_k_add (kernels/pytorch/moe.py:14-37) /
+ * _mul_merge_k_add_fwd (kernels/triton/triton_moe.py:864-914), the second half
+ * of silu_jagged_bmm_combine (kernels/moe.py:236-292).
+ *
+ *   value        [T*K, D], FMOE_BF16 or FMOE_F32, row stride value_stride_row
+ *   gates        logical [gates_rows, gates_cols] read through strides (the
+ *                reference flattens weight.contiguous().view(-1)); dtype
+ *                FMOE_BF16 or FMOE_F32; NULL = unweighted
+ *   out          [T, D] contiguous; dtype = promoted dtype of value and gates
+ */
+int fmoe_combine(const void* value, int value_dtype, int64_t T, int K, int64_t D,
+                 int64_t value_stride_row, const int64_t* reverse_index, const void* gates,
+                 int gates_dtype, int64_t gates_cols, int64_t gates_stride_row,
+                 int64_t gates_stride_col, const int64_t* gates_index, void* out, int out_dtype,
+                 fmoe_stream_t stream);
+
+/* out[i] = silu(a[i]) * b[i] over n bf16 elements with the reference's rounding
+ * points (F.silu(alpha) * beta, kernels/pytorch/moe.py:221): the element-wise
+ * tail of index_select_jagged_gating_bmm when its two inputs differ. */
+int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
+                  fmoe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FAST_MOE_AMD_H */

@@ -1,0 +1,129 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol that
+include/fast_moe_amd.h declares, and rejects bad arguments before touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fast_moe_amd.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from fast_moe_amd.kernels.hip import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from fast_moe_amd import build
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fmoe_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    from fast_moe_amd.kernels.hip import _lib
+    names = declared_functions()
+    assert len(names) >= 9
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert sorted(_lib.EXPORTED_SYMBOLS) == names
+
+
+def test_gemm_desc_layout_matches_header():
+    from fast_moe_amd.kernels.hip._lib import GemmDesc
+    text = open(HEADER).read()
+    body = text[text.index("typedef struct fmoe_gemm_desc {"):text.index("} fmoe_gemm_desc;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = []
+    for stmt in body.split("{", 1)[1].split(";"):
+        stmt = stmt.strip()
+        if not stmt:
+            continue
+        for part in stmt.split(","):
+            name = re.findall(r"([A-Za-z_][A-Za-z0-9_]*)\s*$", part.strip())
+            fields.append(name[0])
+    assert [f[0] for f in GemmDesc._fields_] == fields
+    # sizes and offsets as the C compiler lays them out
+    import subprocess
+    import tempfile
+    prog = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void) {',
+            '  printf("%zu\\n", sizeof(fmoe_gemm_desc));']
+    prog += [f'  printf("%zu\\n", offsetof(fmoe_gemm_desc, {f}));' for f in fields]
+    prog += ['  return 0;', '}']
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "layout.c")
+        open(src, "w").write("\n".join(prog))
+        exe = os.path.join(tmp, "layout")
+        subprocess.run(["gcc", src, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
+    assert int(out[0]) == ctypes.sizeof(GemmDesc)
+    assert [int(v) for v in out[1:]] == [getattr(GemmDesc, f).offset for f in fields]
+
+
+def test_version_and_workspace(lib):
+    assert lib.fmoe_version() >= 100
+    assert lib.fmoe_route_workspace_bytes(0, 8, 2) > 0
+    small = lib.fmoe_route_workspace_bytes(64, 8, 2)
+    big = lib.fmoe_route_workspace_bytes(16384, 64, 8)
+    assert big > small >= 64 * 2 * 2
+    assert lib.fmoe_route_workspace_bytes(-1, 8, 2) == 0
+
+
+def test_argument_errors_are_reported_without_a_gpu(lib):
+    from fast_moe_amd.kernels.hip._lib import GemmDesc
+    assert lib.fmoe_grouped_gemm(None, None) == 1
+    assert b"desc is NULL" in lib.fmoe_last_error()
+    d = GemmDesc()
+    d.num_experts, d.n, d.k = 4, 0, 8
+    assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
+    assert b"n, k >= 1" in lib.fmoe_last_error()
+    d.n, d.total_rows, d.a_dtype, d.out_dtype = 8, 16, 0, 1
+    assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
+    assert b"bf16 or e4m3" in lib.fmoe_last_error()
+    # routing: K > E, K > 64, workspace too small
+    args = [None] * 7
+    assert lib.fmoe_route_topk(None, 0, 4, 8, 80, 1, *args, None, 0, None) == 1
+    assert b"K=80" in lib.fmoe_last_error()
+    assert lib.fmoe_route_topk(None, 0, 4, 8, 2, 1, *args, ctypes.c_void_p(64), 1, None) == 3
+    assert b"workspace" in lib.fmoe_last_error()
+    # quant: zero columns
+    assert lib.fmoe_quant_rows_e4m3(None, 1, 1, 4, 0, 0, 0, 1, 0, None, 0, 0, 1, None, 0, None) == 1
+    # combine: out dtype must be the promoted dtype
+    assert lib.fmoe_combine(ctypes.c_void_p(64), 1, 4, 2, 8, 8, ctypes.c_void_p(64), ctypes.c_void_p(64), 0, 2,
+                            2, 1, None, ctypes.c_void_p(64), 1, None) == 1
+    assert b"promoted" in lib.fmoe_last_error()
+
+
+def test_pytorch_kernel_is_refused():
+    import torch
+    from fast_moe_amd import FastMoELayer, KernelType
+    from fast_moe_amd.kernels import moe
+    with pytest.raises(NotImplementedError):
+        moe.index_select_jagged_bmm(1, torch.zeros(2, dtype=torch.int64), torch.zeros(1, 1, dtype=torch.int64),
+                                    torch.zeros(1, 8), torch.zeros(1, 8, 8), None, kernel=KernelType.PYTORCH)
+    layer = FastMoELayer(8, 16, 8, 4, kernel=KernelType.PYTORCH)
+    with pytest.raises(NotImplementedError):
+        layer(torch.zeros(1, 2, 8, dtype=torch.bfloat16), 2)
+
+
+def test_cpu_tensors_are_refused():
+    import torch
+    from fast_moe_amd.kernels import moe
+    with pytest.raises(ValueError, match="no CPU path"):
+        moe.mul_merge_k_add(torch.zeros(4, dtype=torch.int64), torch.zeros(2, 2, dtype=torch.int64),
+                            torch.zeros(4, 8))
+
+
+def test_state_dict_layout_matches_reference_names():
+    from fast_moe_amd import FastMoELayer
+    layer = FastMoELayer(16, 32, 8, 4)
+    sd = layer.state_dict()
+    assert set(sd) == {"gate.gate.weight", "gate.gate.bias", "_experts_hidden_w", "_experts_hidden_bias",
+                       "_experts_w", "_experts_bias"}
+    assert tuple(sd["_experts_hidden_w"].shape) == (4, 32, 16)
+    assert tuple(sd["_experts_w"].shape) == (4, 8, 32)

@@ -1,0 +1,265 @@
+"""GPU parity: jagged GEMM operators (bf16 and fp8) against the oracle, through the
+operator API (and therefore the C ABI)."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe as o_moe
+from oracle import moe_fp8 as o_fp8
+from tests.helpers import BF16, assert_bf16_close, dev, make_routing, randn, skewed_topk, uniform
+from oracle import routing as o_routing
+
+pytestmark = pytest.mark.gpu
+
+# kernels/tests/moe_test.py:35-84: default assert_close for bf16 is rtol 1.6e-2, atol 1e-5
+REF_RTOL, REF_ATOL = 1.6e-2, 1e-5
+
+
+def weights(E, K, N, seed, contiguous=True, scale=None):
+    w = uniform((E, K, N), seed) if scale is None else randn((E, K, N), seed, scale=scale)
+    if not contiguous:          # [E, K, N] view of [E, N, K] storage (moe_test.py:223-239)
+        w = w.transpose(1, 2).contiguous().transpose(1, 2)
+    return w
+
+
+GRID = [(L, E, K, Din, Dout) for L, E, K, Din, Dout in itertools.product(
+    [16, 100, 500], [4, 16], [2, 4], [12, 32, 64], [32, 128])]
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout", GRID[::3])
+@pytest.mark.parametrize("contiguous", [True, False])
+@pytest.mark.parametrize("has_bias", [True, False])
+def test_index_select_jagged_bmm_reference_grid(L, E, K, Din, Dout, contiguous, has_bias):
+    from fast_moe_amd.kernels import moe
+    print(f"bmm L={L} E={E} K={K} Din={Din} Dout={Dout} contiguous={contiguous} bias={has_bias}", flush=True)
+    r = make_routing(L, E, K, seed=L + E)
+    x = uniform((L, Din), 1)
+    w = weights(E, Din, Dout, 2, contiguous)
+    b = uniform((E, Dout), 3) if has_bias else None
+    ref = o_moe.index_select_jagged_bmm(r["offsets"], r["index"], x.float(), w.float(),
+                                        None if b is None else b.float())
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm(int(r["lengths"].max()), dev(r["offsets"]), dev(r["index"]), dev(x),
+                                          dev(w), dev(b))
+    assert out.dtype == BF16 and tuple(out.shape) == (L * K, Dout)
+    torch.testing.assert_close(out.cpu(), ref.to(BF16), rtol=REF_RTOL, atol=REF_ATOL)
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,contiguous", [
+    (2048, 8, 2, 256, 512, False),      # tall tiles, K-contiguous weights (the layer's layout)
+    (2048, 8, 2, 256, 512, True),       # tall tiles, N-contiguous weights
+    (1500, 4, 2, 200, 136, False),      # ragged rows, K tail, N tail
+    (4096, 64, 8, 128, 96, False),
+    (300, 128, 8, 64, 256, False),      # short tiles
+])
+def test_index_select_jagged_bmm_larger(L, E, K, Din, Dout, contiguous):
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=L)
+    x = randn((L, Din), 1)
+    w = weights(E, Din, Dout, 2, contiguous, scale=Din ** -0.5)
+    b = randn((E, Dout), 3)
+    ref = o_moe.index_select_jagged_bmm(r["offsets"], r["index"], x.float(), w.float(), b.float())
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b))
+    assert_bf16_close(out, ref, rtol=1e-2, atol=1e-2, what="index_select_jagged_bmm")
+
+
+def test_skewed_and_empty_experts():
+    from fast_moe_amd.kernels import moe
+    T, E, K, D, H = 4096, 64, 8, 128, 192
+    topk = skewed_topk(T, E, K, seed=3)
+    meta = o_routing.routing_metadata(topk.numpy(), E)
+    assert (meta["lengths"] == 0).sum() >= 2 and meta["lengths"].max() > 8 * meta["lengths"][meta["lengths"] > 0].min()
+    offsets = torch.from_numpy(meta["offsets"])
+    index = torch.from_numpy(meta["gate_index"]).view(-1, K)
+    x = randn((T, D), 1)
+    wg = weights(E, D, H, 2, False, scale=D ** -0.5)
+    wu = weights(E, D, H, 3, False, scale=D ** -0.5)
+    ref = o_moe.index_select_jagged_bmm_swiglu(offsets, index, x.float(), wg.float(), None, wu.float(), None)
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm_swiglu(0, dev(offsets), dev(index), dev(x), dev(wg), None, dev(wu), None)
+    assert_bf16_close(out, ref, what="swiglu, skewed")
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,bias,contiguous", [
+    (100, 8, 2, 32, 64, True, True), (500, 4, 4, 64, 64, False, False), (2048, 8, 2, 128, 256, True, False),
+    (64, 16, 2, 24, 40, True, True)])
+def test_swiglu_and_gating(L, E, K, Din, Dout, bias, contiguous):
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=L + 1)
+    x, x2 = uniform((L, Din), 1), uniform((L, Din), 4)
+    w, wp = weights(E, Din, Dout, 2, contiguous), weights(E, Din, Dout, 5, contiguous)
+    b = uniform((E, Dout), 3) if bias else None
+    bp = uniform((E, Dout), 6) if bias else None
+    f = lambda t: None if t is None else t.float()
+    ref = o_moe.index_select_jagged_bmm_swiglu(r["offsets"], r["index"], f(x), f(w), f(b), f(wp), f(bp))
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm_swiglu(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b),
+                                                 dev(wp), dev(bp))
+        xa = dev(x)
+        out_same = moe.index_select_jagged_gating_bmm(0, dev(r["offsets"]), dev(r["index"]), xa, xa, dev(w),
+                                                      dev(b), dev(wp), dev(bp))
+        out_two = moe.index_select_jagged_gating_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(x2),
+                                                     dev(w), dev(b), dev(wp), dev(bp))
+    # tolerance of kernels/tests/moe_test.py:729-949 for bf16 products of two GEMMs
+    assert_bf16_close(out, ref, rtol=1.6e-2, atol=2e-2, what="swiglu")
+    assert torch.equal(out, out_same)
+    ref2 = o_moe.index_select_jagged_gating_bmm(r["offsets"], r["index"], f(x), f(x2), f(w), f(wp), f(b), f(bp))
+    assert_bf16_close(out_two, ref2, rtol=1.6e-2, atol=2e-2, what="gating")
+
+
+def test_3d_variant():
+    from fast_moe_amd.kernels import moe
+    L, E, K, Din, Dout = 200, 4, 2, 8, 4
+    r = make_routing(L, E, K, seed=9)
+    x = uniform((L, E, Din), 1)
+    w = weights(E, Din, Dout, 2)
+    b = uniform((E, Dout), 3)
+    ref = o_moe.index_select_jagged_bmm_3D(r["offsets"], r["index"], x.float(), w.float(), b.float())
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm_3D(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b))
+    torch.testing.assert_close(out.cpu(), ref.to(BF16), rtol=REF_RTOL, atol=REF_ATOL)
+    L, Din, Dout = 600, 64, 64
+    r = make_routing(L, E, K, seed=10)
+    x = uniform((L, E, Din), 1)
+    w = weights(E, Din, Dout, 2, contiguous=False)
+    ref = o_moe.index_select_jagged_bmm_3D(r["offsets"], r["index"], x.float(), w.float(), None)
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm_3D(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), None)
+    torch.testing.assert_close(out.cpu(), ref.to(BF16), rtol=REF_RTOL, atol=1e-4)
+
+
+@pytest.mark.parametrize("E,K,Din,Dout,has_silu,has_bias,max_len", [
+    (4, 1, 128, 128, True, True, 64), (8, 2, 256, 128, False, True, 200), (8, 2, 128, 256, True, False, 200),
+    (4, 2, 256, 256, False, False, 32), (8, 2, 1024, 512, True, True, 700)])
+def test_silu_jagged_bmm_combine(E, K, Din, Dout, has_silu, has_bias, max_len):
+    """Generator of kernels/tests/moe_test.py:1017-1032; tolerance far inside its atol 5e-1 / rtol 1.5e-1."""
+    from fast_moe_amd.kernels import moe
+    g = torch.Generator().manual_seed(E + K + Din)
+    seq_len = torch.randint(32, max_len + 1, (E,), generator=g)
+    N = int(seq_len.sum())
+    logits = (torch.rand(N, E, generator=g) + 1e-2).to(BF16)
+    topk_gates, topk_idx = logits.topk(K, dim=1)
+    meta = o_routing.routing_metadata(topk_idx.numpy(), E)
+    t = lambda k: torch.from_numpy(meta[k])
+    jagged = uniform((N * K, Din), 1)
+    w = weights(E, Din, Dout, 2)
+    b = uniform((E, Dout), 3) if has_bias else None
+    ref = o_moe.silu_jagged_bmm_combine(t("offsets"), jagged, w, b, t("token_index"), K, topk_gates,
+                                        t("gate_index"), has_silu)
+    ref32 = o_moe.silu_jagged_bmm_combine(
+        t("offsets"), (torch.nn.functional.silu(jagged) if has_silu else jagged).float(), w.float(),
+        None if b is None else b.float(), t("token_index"), K, topk_gates.float(), t("gate_index"), False)
+    with torch.no_grad():
+        out = moe.silu_jagged_bmm_combine(0, dev(t("offsets")), dev(jagged), dev(w), dev(b), dev(t("token_index")),
+                                          dev(t("reverse_index")), dev(topk_gates), dev(t("gate_index")),
+                                          has_silu=has_silu)
+    assert out.dtype == BF16 and tuple(out.shape) == (N, Dout)
+    assert_bf16_close(out, ref32, rtol=2e-2, atol=5e-2 * (Din / 128) ** 0.5, what="combine vs fp32")
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=5e-1, rtol=1.5e-1)
+
+
+@pytest.mark.parametrize("N,K,D,dtype,wdtype", [
+    (2, 4, 128, torch.float32, torch.float32), (33, 16, 256, BF16, BF16), (100, 32, 128, BF16, BF16),
+    (1000, 4, 256, torch.float32, torch.float32), (512, 8, 2048, BF16, BF16), (64, 3, 100, BF16, BF16),
+    (40, 5, 37, torch.float32, torch.float32), (128, 8, 512, BF16, torch.float32)])
+def test_mul_merge_k_add_bit_exact(N, K, D, dtype, wdtype):
+    """Generator of kernels/tests/moe_test.py:344-367: non-contiguous weight, permuted weight_index,
+    arbitrary row -> output map.  The fp32 adds follow the CPU index_add order, so the result is
+    bit-identical to the oracle."""
+    from fast_moe_amd.kernels import moe
+    g = torch.Generator().manual_seed(N + K)
+    x = uniform((N * K, D), 1, dtype)
+    w = uniform((N, 2 * K), 2, wdtype)[:, :K]
+    w_index = torch.randperm(N * K, generator=g)
+    perm = torch.randperm(N * K, generator=g)
+    o2i = torch.arange(N).repeat(K)[perm]
+    i2o = o2i.sort(stable=True)[1].view(-1, K)
+    ref = o_moe.mul_merge_k_add(o2i, x, K, w, w_index)
+    with torch.no_grad():
+        out = moe.mul_merge_k_add(dev(o2i), dev(i2o), dev(x), weight=dev(w), weight_index=dev(w_index))
+        out_nw = moe.mul_merge_k_add(dev(o2i), dev(i2o), dev(x))
+    assert out.dtype == ref.dtype
+    assert torch.equal(out.cpu(), ref), f"max diff {(out.cpu().float() - ref.float()).abs().max()}"
+    assert torch.equal(out_nw.cpu(), o_moe.mul_merge_k_add(o2i, x, K))
+
+
+# ------------------------------------------------------------------------ fp8
+@pytest.mark.parametrize("L,E,K,Din,Dout,bias,contiguous", [
+    (16, 4, 2, 32, 16, True, True), (100, 8, 4, 64, 32, False, True), (500, 16, 2, 64, 16, True, False),
+    (2048, 8, 2, 256, 512, True, False), (300, 4, 2, 48, 24, True, True), (4096, 64, 8, 256, 128, False, False)])
+def test_fp8_gather_gemm(L, E, K, Din, Dout, bias, contiguous):
+    """kernels/tests/moe_fp8_test.py:337-370: fp8 kernel vs the PyTorch fp8 emulation, 1e-2 / 1e-2."""
+    from fast_moe_amd.kernels import moe_fp8
+    r = make_routing(L, E, K, seed=L + 2)
+    x = uniform((L, Din), 1)
+    w = weights(E, Din, Dout, 2, contiguous)
+    b = uniform((E, Dout), 3) if bias else None
+    ref = o_fp8.index_select_jagged_bmm_fp8(r["offsets"], r["index"], x, w, b)
+    with torch.no_grad():
+        out = moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b),
+                                              fp8=True)
+        raw = moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b),
+                                              fp8=False)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), atol=1e-2, rtol=1e-2)
+    # vs the unquantised op: tolerance of moe_fp8_test.py:302-335
+    torch.testing.assert_close(out.cpu().float(), raw.cpu().float(), atol=4e-1, rtol=1e-1)
+
+
+def test_fp8_outlier_rows_and_zero_rows():
+    from fast_moe_amd.kernels import moe_fp8
+    L, E, K, Din, Dout = 512, 8, 2, 128, 64
+    r = make_routing(L, E, K, seed=4)
+    x = randn((L, Din), 1)
+    x[::50] *= 100
+    x[7] = 0
+    w = weights(E, Din, Dout, 2, False, scale=Din ** -0.5)
+    w[3, :, 5] = 0
+    ref = o_fp8.index_select_jagged_bmm_fp8(r["offsets"], r["index"], x, w, None)
+    with torch.no_grad():
+        out = moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), None, fp8=True)
+    assert bool(torch.isfinite(out).all())
+    err = (out.cpu().float() - ref.float()).abs()
+    assert bool((err <= 3e-2 * ref.float().abs() + 3e-2).all())
+
+
+@pytest.mark.parametrize("E,K,Din,Dout,has_silu", [(4, 2, 128, 128, True), (8, 2, 256, 64, False)])
+def test_fp8_combine(E, K, Din, Dout, has_silu):
+    from fast_moe_amd.kernels import moe_fp8
+    g = torch.Generator().manual_seed(E)
+    N = 300
+    logits = (torch.rand(N, E, generator=g) + 1e-2).to(BF16)
+    gates, topk_idx = logits.topk(K, dim=1)
+    meta = o_routing.routing_metadata(topk_idx.numpy(), E)
+    t = lambda k: torch.from_numpy(meta[k])
+    jagged = uniform((N * K, Din), 1)
+    w = weights(E, Din, Dout, 2)
+    b = uniform((E, Dout), 3)
+    # oracle: the same fp8 emulation for the GEMM, then the merge
+    h = torch.nn.functional.silu(jagged) if has_silu else jagged
+    qa, sa = o_fp8.rowwise_quant_fp8(h)
+    qw, sw = o_fp8.rowwise_quant_fp8(w.permute(0, 2, 1))
+    sizes = (t("offsets")[1:] - t("offsets")[:-1]).tolist()
+    rows = o_fp8.fp8_linear_per_expert(list(o_fp8.dequant(qa).split(sizes)), list(sa.split(sizes)),
+                                       o_fp8.dequant(qw), sw, b, BF16)
+    ref = o_moe.mul_merge_k_add(t("token_index"), torch.cat(rows), K, gates, t("gate_index"))
+    with torch.no_grad():
+        out = moe_fp8.silu_jagged_bmm_combine_fp8(0, dev(t("offsets")), dev(jagged), dev(w), dev(b),
+                                                  dev(t("token_index")), dev(t("reverse_index")), dev(gates),
+                                                  dev(t("gate_index")), has_silu=has_silu)
+    err = (out.cpu().float() - ref.float()).abs()
+    assert bool((err <= 3e-2 * ref.float().abs() + 3e-2).all()), err.max()
+
+
+def test_forward_only_and_dtype_errors():
+    from fast_moe_amd.kernels import moe
+    r = make_routing(16, 4, 2)
+    x = uniform((16, 32), 1).cuda().requires_grad_()
+    w = weights(4, 32, 32, 2).cuda()
+    with pytest.raises(RuntimeError, match="forward-only"):
+        moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, None)
+    with pytest.raises(NotImplementedError):
+        with torch.no_grad():
+            moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x.float(), w.float(), None)
