@@ -3,6 +3,20 @@
 
 using namespace fmoe;
 
+namespace fmoe {
+int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+}  // namespace fmoe
+
 extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_) {
     hipStream_t stream = (hipStream_t)stream_;
     FMOE_REQUIRE(d != nullptr, "fmoe_grouped_gemm: desc is NULL");
@@ -38,6 +52,9 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     p.N = d->n;
     p.K = d->k;
     p.index_div = d->index_div;
+    p.index_shift = -1;
+    for (int s = 0; s < 31; ++s)
+        if (d->index_div == (1 << s)) p.index_shift = s;
     p.total_rows = d->total_rows;
     p.a_rows = d->a_rows;
     p.a = (const uint8_t*)d->a;
@@ -57,8 +74,7 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     p.out = (uint16_t*)d->out;
     p.out_stride = d->out_stride_row;
     p.n_tiles = 0;
-    p.vec_store = (d->n % 4 == 0) && (d->out_stride_row % 4 == 0) &&
-                  ((reinterpret_cast<uintptr_t>(d->out) & 7u) == 0);
+    p.vec_store = (d->n % 8 == 0) && (d->out_stride_row % 8 == 0) && aligned16(d->out);
 
     const int esize = fp8 ? 1 : 2;
     const int chunk = 16 / esize;
@@ -69,6 +85,11 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     // rows per expert decide the tile height: tall tiles for prefill-like loads,
     // short ones when the experts see a handful of rows (weight-streaming regime)
     const bool big = d->total_rows / d->num_experts >= 96;
-    if (fp8) return run_gemm_fp8(p, d->epilogue, fast, big, stream);
-    return run_gemm_bf16(p, d->epilogue, d->a_silu != 0, fast, big, stream);
+    // the ring kernel moves whole 64-byte K-slices by LDS-DMA and stores 16-byte groups
+    const int slice = 64 / esize;
+    const bool ring = fast && big && !d->a_silu && (d->k % slice) == 0 && d->k / slice >= 3 &&
+                      p.vec_store && d->num_experts <= 1024 && d->total_rows < ((int64_t)1 << 31) * 128;
+    const int sel = !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
+    if (fp8) return run_gemm_fp8(p, d->epilogue, sel, stream);
+    return run_gemm_bf16(p, d->epilogue, d->a_silu != 0, sel, stream);
 }

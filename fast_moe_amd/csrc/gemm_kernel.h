@@ -2,35 +2,47 @@
 // bf16 or OCP-e4m3 operands, fp32 MFMA accumulation, fused bias / SiLU / SwiGLU
 // epilogue.  Shared by gemm_bf16.hip and gemm_fp8.hip.
 //
+// Two kernels share the tile geometry, the scheduler and the epilogue:
+//
+//   grouped_gemm_ring_kernel   the fast path.  Persistent (one block per CU), 256 x 256 tiles,
+//       8 wavefronts.  Operand K-slices of 64 bytes per row travel global -> LDS with
+//       global_load_lds_dwordx4 (no VGPR staging) into a 4-slot ring, three slices in flight
+//       per CU; the ring runs across tile boundaries, so the loads of the next tile are
+//       already under way while the current tile's epilogue stores drain.
+//   grouped_gemm_kernel        register-staged, double-buffered LDS; serves everything the
+//       ring kernel does not: arbitrary B strides and K / N tails (element loads), SiLU
+//       applied to A on load, and short 64-row tiles for experts with a handful of rows.
+//
 // Mapping to the hardware
-//   * A tile is BM activation rows x BN weight rows; both operands are staged as
-//     128-byte K-slices per row (64 bf16 or 128 e4m3) in double-buffered LDS,
-//     16-byte chunks XOR-swizzled by (row >> 1) & 7 so that the ds_read_b128 of
-//     an MFMA fragment and the ds_write_b128 of the loader spread over all banks.
+//   * LDS rows are XOR-swizzled in 16-byte chunks so that the ds_read_b128 of an MFMA
+//     fragment is conflict free; for the ring kernel the swizzle is applied by permuting
+//     which global chunk each lane fetches, because LDS-DMA lays lanes out linearly.
 //   * The weights feed the MFMA "A" port and the activations the "B" port
-//     (v_mfma_f32_32x32x16_bf16 / v_mfma_f32_32x32x64_f8f6f4), so each lane ends
-//     up with 4 consecutive output columns of one output row per register quad
-//     and stores them as one 8-byte write.
-//   * Activation rows are gathered through row_index while loading (no [R, K]
-//     copy); rows past the end of an expert segment re-read the tile's first row
-//     and are masked at the store.
-//   * Scheduling is on the device: every block derives the number of row tiles
-//     per expert from `offsets` with a wavefront prefix scan, so no max_seq_len
-//     and no host synchronisation are needed, skewed and empty experts cost
-//     nothing, and the grid is only an upper bound.  Block ids are dealt
-//     round-robin to the 8 XCDs by the hardware; id -> tile is remapped so that
-//     each XCD works on a contiguous range of tiles (group-of-4 row tiles x all
-//     column tiles), which keeps the shared A rows / B rows in that XCD's L2.
+//     (v_mfma_f32_32x32x16_bf16 / v_mfma_f32_32x32x64_f8f6f4), so a lane holds 4 consecutive
+//     output columns of one output row per register quad; v_permlane32_swap pairs two
+//     quads into 16 contiguous bytes for the store.
+//   * Activation rows are gathered through row_index while loading (no [R, K] copy); rows
+//     past the end of an expert segment re-read the tile's first row and are masked at the
+//     store.
+//   * Scheduling is on the device: the number of row tiles per expert comes from `offsets`
+//     (wavefront prefix scan), so no max_seq_len and no host synchronisation are needed and
+//     skewed or empty experts cost nothing.  Block ids are dealt round-robin to the 8 XCDs by
+//     the hardware; id -> tile is remapped so that each XCD works on a contiguous range of
+//     tiles (groups of 4 row tiles x all column tiles), which keeps shared rows in its L2.
 #pragma once
 
 #include "common.h"
 
 namespace fmoe {
 
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+
 struct GemmParams {
     const int64_t* offsets;
     const int64_t* row_index;
     int E, N, K, index_div;
+    int index_shift;                    // log2(index_div) when it is a power of two, else -1
     int64_t total_rows, a_rows;
     const uint8_t* a;
     int64_t a_stride_row, a_stride_e;   // elements
@@ -46,9 +58,138 @@ struct GemmParams {
     uint16_t* out;
     int64_t out_stride;
     int n_tiles;
-    int vec_store;                      // 8-byte stores of 4 bf16 are legal
+    int vec_store;                      // 16-byte stores of 8 bf16 are legal
 };
 
+constexpr int kGroupM = 4;   // row tiles per scheduling group
+constexpr int kNumXcd = 8;
+
+__device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) {
+    return v < lo ? lo : (v > hi ? hi : v);
+}
+
+__device__ __forceinline__ int64_t source_row(const GemmParams& p, int64_t r) {
+    int64_t s = r;
+    if (p.row_index) {
+        const int64_t v = p.row_index[r];
+        s = p.index_shift >= 0 ? (v >> p.index_shift) : v / p.index_div;
+    }
+    return clamp_i64(s, 0, p.a_rows - 1);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {   // v_cvt_pk_bf16_f32, RNE
+    f32x2 v = {a, b};
+    bf16x2 r = __builtin_convertvector(v, bf16x2);
+    return *reinterpret_cast<uint32_t*>(&r);
+}
+__device__ __forceinline__ float rbf(float a) {   // round to bf16 and back
+    return (float)(__bf16)a;
+}
+
+// SiLU on 8 packed bf16 with the rounding of F.silu on a bf16 tensor
+__device__ __forceinline__ u32x4 silu_bf16x8(u32x4 v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = silu_f32(bf16_bits_to_f32(v[j] & 0xffffu));
+        const float hi = silu_f32(__uint_as_float(v[j] & 0xffff0000u));
+        v[j] = pack_bf16(lo, hi);
+    }
+    return v;
+}
+
+// ------------------------------------------------------------------------ epilogue
+// acc[fn][fm][v]: fragment (fn, fm) of the wave tile, v = 4*g + j <-> output row
+// (lane & 31) of fragment row block fm, output column 32*fn + 8*g + 4*(lane >> 5) + j.
+// Rounding points follow the reference's bf16 path: GEMM result (+bias) rounded to bf16,
+// SiLU rounded to bf16, product rounded to bf16; e4m3 operands: (acc / (s_a * s_w)) rounded,
+// then the bias added in bf16.
+template <int FM, int FN, int TM, int TN, bool FP8, int EPI>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
+                                              int n0, int64_t row0, int rows_valid, int wm, int wn,
+                                              int lane) {
+    constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
+    constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
+    const int khalf = lane >> 5;
+    const int64_t bias_row = (int64_t)expert * p.bias_se;
+    float rsa[FM];
+    bool row_ok[FM];
+    uint16_t* orow[FM];
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+        const int tile_row = wm * TM + fm * 32 + (lane & 31);
+        row_ok[fm] = tile_row < rows_valid;
+        orow[fm] = p.out + (row0 + tile_row) * p.out_stride;
+        rsa[fm] = 1.0f;
+        if (FP8) rsa[fm] = 1.0f / p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))];
+    }
+#pragma unroll
+    for (int fn = 0; fn < FN_OUT; ++fn) {
+#pragma unroll
+        for (int gp = 0; gp < 2; ++gp) {
+            // register quads g = 2gp and 2gp+1: columns nq + 8*q + 4*khalf + j
+            const int nq = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + fn * 32 + 16 * gp;
+            float rsw[2][4], rsw2[2][4], bv[2][4], bv2[2][4];
+#pragma unroll
+            for (int q = 0; q < 2; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = nq + 8 * q + 4 * khalf + j;
+                    const int nc = n < p.N ? n : p.N - 1;
+                    rsw[q][j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                    rsw2[q][j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                    bv[q][j] = p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
+                    bv2[q][j] = (SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
+                }
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) {
+                float o[2][4];
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int v = 4 * (2 * gp + q) + j;
+                        float y = acc[fn][fm][v];
+                        float y2 = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
+                        if (FP8) {
+                            y = rbf(y * (rsa[fm] * rsw[q][j]));
+                            if (p.bias) y = rbf(y + bv[q][j]);
+                            if (SWIGLU) {
+                                y2 = rbf(y2 * (rsa[fm] * rsw2[q][j]));
+                                if (p.bias2) y2 = rbf(y2 + bv2[q][j]);
+                            }
+                        } else {
+                            y = rbf(y + bv[q][j]);
+                            if (SWIGLU) y2 = rbf(y2 + bv2[q][j]);
+                        }
+                        if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
+                        if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
+                        o[q][j] = y;
+                    }
+                if (p.vec_store) {
+                    // pair the quads of the two lane halves: low lanes end up with columns
+                    // nq..nq+7, high lanes with nq+8..nq+15 of their row
+                    const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][0], o[0][1]),
+                                                                      pack_bf16(o[1][0], o[1][1]), false, false);
+                    const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][2], o[0][3]),
+                                                                      pack_bf16(o[1][2], o[1][3]), false, false);
+                    const int nb = nq + 8 * khalf;
+                    if (row_ok[fm] && nb + 7 < p.N)
+                        *reinterpret_cast<u32x4*>(orow[fm] + nb) = u32x4{s0[0], s1[0], s0[1], s1[1]};
+                } else if (row_ok[fm]) {
+#pragma unroll
+                    for (int q = 0; q < 2; ++q)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int n = nq + 8 * q + 4 * khalf + j;
+                            if (n < p.N) orow[fm][n] = (uint16_t)f32_to_bf16_bits(o[q][j]);
+                        }
+                }
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------- register-staged kernel
 template <int BM_, int BN_, int WGM_, int WGN_>
 struct TileCfg {
     static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_;
@@ -61,26 +202,8 @@ struct TileCfg {
     static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0, "loader passes must be whole");
 };
 
-constexpr int kGroupM = 4;   // row tiles per scheduling group
-constexpr int kNumXcd = 8;
-
-__device__ __forceinline__ int lds_off(int row, int chunk) {
+__device__ __forceinline__ int lds_off(int row, int chunk) {     // 128-byte rows
     return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4);
-}
-
-__device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) {
-    return v < lo ? lo : (v > hi ? hi : v);
-}
-
-// SiLU on 8 packed bf16 with the rounding of F.silu on a bf16 tensor
-__device__ __forceinline__ u32x4 silu_bf16x8(u32x4 v) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const float lo = round_bf16(silu_f32(bf16_bits_to_f32(v[j] & 0xffffu)));
-        const float hi = round_bf16(silu_f32(__uint_as_float(v[j] & 0xffff0000u)));
-        v[j] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
-    }
-    return v;
 }
 
 template <typename TL, bool FP8, int EPI, bool FAST, bool A_SILU>
@@ -168,10 +291,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
     const int n0 = nt * BN_OUT;
 
     auto src_row_of = [&](int tile_row) -> int64_t {
-        const int64_t r = row0 + (tile_row < rows_valid ? tile_row : 0);
-        int64_t s = r;
-        if (p.row_index) s = p.row_index[r] / p.index_div;
-        return clamp_i64(s, 0, p.a_rows - 1);
+        return source_row(p, row0 + (tile_row < rows_valid ? tile_row : 0));
     };
     // weight row (output column) behind LDS row `wrow`, and which matrix holds it
     auto w_row_of = [&](int wrow, const uint8_t*& base) -> int {
@@ -216,12 +336,14 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
 
     u32x4 xr[XP], wr[WP];
     auto load_global = [&](int kt) {
+        const bool whole = (kt + 1) * BK <= p.K;      // uniform: no per-lane predicate inside K
 #pragma unroll
         for (int i = 0; i < XP; ++i) {
             const int k = kt * BK + xchunk[i] * CHUNK_ELEMS;
             if (FAST) {
-                xr[i] = k < p.K ? *reinterpret_cast<const u32x4*>(xptr[i] + (int64_t)k * ESIZE)
-                                : u32x4{0, 0, 0, 0};
+                if (whole) xr[i] = *reinterpret_cast<const u32x4*>(xptr[i] + (int64_t)k * ESIZE);
+                else xr[i] = k < p.K ? *reinterpret_cast<const u32x4*>(xptr[i] + (int64_t)k * ESIZE)
+                                     : u32x4{0, 0, 0, 0};
             } else {
                 uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -240,8 +362,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
         for (int i = 0; i < WP; ++i) {
             const int k = kt * BK + wchunk[i] * CHUNK_ELEMS;
             if (FAST) {
-                wr[i] = k < p.K ? *reinterpret_cast<const u32x4*>(wptr[i] + (int64_t)k * ESIZE)
-                                : u32x4{0, 0, 0, 0};
+                if (whole) wr[i] = *reinterpret_cast<const u32x4*>(wptr[i] + (int64_t)k * ESIZE);
+                else wr[i] = k < p.K ? *reinterpret_cast<const u32x4*>(wptr[i] + (int64_t)k * ESIZE)
+                                     : u32x4{0, 0, 0, 0};
             } else {
                 uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -345,78 +468,332 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
         __syncthreads();
     }
 
-    // -------------------------------------------------------------- epilogue
-    // Register quad g of fragment (fn, fm) holds output columns nb .. nb+3 of row
-    // (lane & 31) of the fragment.  Per-column data (weight descale, bias) is
-    // fetched once per quad and reused over the FM row fragments.
-    constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
-    const int64_t bias_row = (int64_t)expert * p.bias_se;
-    float rsa[FM];
-    bool row_ok[FM];
-    uint16_t* orow[FM];
+    gemm_epilogue<FM, FN, TM, TN, FP8, EPI>(p, acc, expert, n0, row0, rows_valid, wm, wn, lane);
+}
+
+// --------------------------------------------------------------------- ring kernel
+template <int BM_, int BN_, int WGM_, int WGN_, int STAGES_>
+struct RingCfg {
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_, STAGES = STAGES_;
+    static constexpr int NW = WGM * WGN;
+    static constexpr int NT = kWave * NW;
+    static constexpr int TM = BM / WGM, TN = BN / WGN;
+    static constexpr int FM = TM / 32, FN = TN / 32;
+    static constexpr int STAGE_BYTES = (BM + BN) * 64;          // 64-byte K-slice per row
+    static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+    static constexpr int kMaxExperts = 1024;
+    static constexpr int TAB_OFF = RING_BYTES;                   // int32 [E+1] row-tile prefix
+    static constexpr int OFF_OFF = RING_BYTES + 4128;            // int64 [E+1] clamped offsets
+    static constexpr int LDS_BYTES = OFF_OFF + (kMaxExperts + 1) * 8 + 8;
+    static constexpr int XI = BM / 16 / NW, WI = BN / 16 / NW;   // LDS-DMA instructions per lane per slice
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "DMA passes must be whole");
+    static_assert(STAGES == 3 || STAGES == 4, "the wait ladder below covers 3 or 4 slots");
+    static_assert(TM % 32 == 0 && TN % 64 == 0, "wave tile must hold whole 32x32 fragments, FN even");
+};
+
+__device__ __forceinline__ int lds_off64(int row, int chunk) {   // 64-byte rows
+    return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4);
+}
+
+// One 16-byte-per-lane global -> LDS transfer.  The 64 lanes land on 1 KB of LDS starting at
+// the wave-uniform byte address lds_addr (M0), lane l at +16*l.  Issued as inline asm so
+// that the waits on it stay under this kernel's control (vmcnt is counted by hand below).
+__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n"
+                 :: "v"(gptr), "s"(lds_addr) : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+template <typename TL, bool FP8, int EPI>
+__global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmParams p) {
+    constexpr int BM = TL::BM, BN = TL::BN, NW = TL::NW, STAGES = TL::STAGES;
+    constexpr int FM = TL::FM, FN = TL::FN, TM = TL::TM, TN = TL::TN;
+    constexpr int ESIZE = FP8 ? 1 : 2;
+    constexpr int BK = 64 / ESIZE;
+    constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
+    constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
+    constexpr int XI = TL::XI, WI = TL::WI;
+    constexpr int L = XI + WI;
+
+    extern __shared__ __align__(16) uint8_t smem[];
+    int32_t* s_tab = reinterpret_cast<int32_t*>(smem + TL::TAB_OFF);   // [E+1] row-tile prefix
+    int64_t* s_off = reinterpret_cast<int64_t*>(smem + TL::OFF_OFF);   // [E+1] clamped offsets
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % TL::WGM, wn = wave / TL::WGM;
+    const int khalf = lane >> 5;
+
+    // ------------------------------------------------------------ schedule tables
+    const int64_t R = p.total_rows;
+    if (wave == 0) {
+        int run = 0;
+        for (int e0 = 0; e0 <= p.E; e0 += kWave) {
+            const int e = e0 + lane;
+            int64_t lo = 0, len = 0;
+            if (e <= p.E) lo = clamp_i64(p.offsets[e], 0, R);
+            if (e < p.E) {
+                const int64_t hi = clamp_i64(p.offsets[e + 1], 0, R);
+                len = hi > lo ? hi - lo : 0;
+            }
+            const int tiles = (int)((len + BM - 1) / BM);
+            const int inc = wave_inclusive_scan(tiles);
+            if (e < p.E) s_tab[e + 1] = run + inc;
+            if (e <= p.E) s_off[e] = lo;
+            run += wave_bcast(inc, kWave - 1);
+        }
+        if (lane == 0) s_tab[0] = 0;
+    }
+    __syncthreads();
+    const int total_m = s_tab[p.E];
+    const int64_t total_tiles = (int64_t)total_m * p.n_tiles;
+    const int nslots = gridDim.x / kNumXcd;
+    const int64_t per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
+    const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+    const int64_t xcd_begin = xcd * per_xcd;
+    int64_t xcd_end = xcd_begin + per_xcd;
+    if (xcd_end > total_tiles) xcd_end = total_tiles;
+
+    struct TileInfo { int expert; int nt; int64_t row0; int rows_valid; };
+    auto locate = [&](int64_t logical) -> TileInfo {
+        const int64_t group_span = (int64_t)kGroupM * p.n_tiles;
+        const int64_t group = logical / group_span;
+        const int first_m = (int)(group * kGroupM);
+        const int gsize = total_m - first_m < kGroupM ? total_m - first_m : kGroupM;
+        const int within = (int)(logical - group * group_span);
+        const int mt = first_m + within % gsize;
+        TileInfo t;
+        t.nt = within / gsize;
+        int lo = 0, hi = p.E;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_tab[mid] <= mt) lo = mid; else hi = mid;
+        }
+        t.expert = lo;
+        const int64_t e_lo = s_off[lo], e_hi = s_off[lo + 1];
+        t.row0 = e_lo + (int64_t)(mt - s_tab[lo]) * BM;
+        const int64_t left = (e_hi > e_lo ? e_hi : e_lo) - t.row0;
+        t.rows_valid = (int)(left < BM ? left : BM);
+        return t;
+    };
+
+    // ------------------------------------------------------------ LDS-DMA geometry
+    // DMA instruction i of this wave fills LDS rows (i*NW + wave)*16 .. +15 of the X (or W)
+    // part of a ring slot: lane l -> row + l/4, 16-byte position l%4, which holds global
+    // chunk (l%4) ^ ((row >> 2) & 3) of that row's 64-byte K-slice (the read-side swizzle).
+    int xrow[XI], wrow[WI];
+    int xsw[XI], wsw[WI];
 #pragma unroll
-    for (int fm = 0; fm < FM; ++fm) {
-        const int tile_row = wm * TM + fm * 32 + (lane & 31);
-        row_ok[fm] = tile_row < rows_valid;
-        orow[fm] = p.out + (row0 + tile_row) * p.out_stride;
-        rsa[fm] = FP8 ? 1.0f / p.a_scale[src_row_of(tile_row)] : 1.0f;
+    for (int i = 0; i < XI; ++i) {
+        xrow[i] = (i * NW + wave) * 16 + (lane >> 2);
+        xsw[i] = (((lane & 3) ^ ((xrow[i] >> 2) & 3)) << 4);
     }
 #pragma unroll
-    for (int fn = 0; fn < FN_OUT; ++fn) {
+    for (int i = 0; i < WI; ++i) {
+        wrow[i] = (i * NW + wave) * 16 + (lane >> 2);
+        wsw[i] = (((lane & 3) ^ ((wrow[i] >> 2) & 3)) << 4);
+    }
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem;
+
+    // source rows (row_index entries) of a tile, fetched ahead of the pointer computation
+    auto fetch_rows = [&](const TileInfo& t, int64_t* ridx) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int nb = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + fn * 32 + 8 * g + 4 * khalf;
-            float rsw[4], rsw2[4], bv[4], bv2[4];
+        for (int i = 0; i < XI; ++i) {
+            const int64_t r = t.row0 + (xrow[i] < t.rows_valid ? xrow[i] : 0);
+            ridx[i] = p.row_index ? p.row_index[r] : r;
+        }
+    };
+    const uint8_t* xptr[XI];
+    const uint8_t* wptr[WI];
+    auto make_ptrs = [&](const TileInfo& t, const int64_t* ridx) {
+        const uint8_t* a_base = p.a + (int64_t)t.expert * p.a_stride_e * ESIZE;
+        const int n0 = t.nt * BN_OUT;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int nc = nb + j < p.N ? nb + j : p.N - 1;
-                rsw[j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                rsw2[j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                bv[j] = p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
-                bv2[j] = (SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
+        for (int i = 0; i < XI; ++i) {
+            int64_t s = ridx[i];
+            if (p.row_index) s = p.index_shift >= 0 ? (s >> p.index_shift) : s / p.index_div;
+            s = clamp_i64(s, 0, p.a_rows - 1);
+            xptr[i] = a_base + s * (p.a_stride_row * ESIZE) + xsw[i];
+        }
+#pragma unroll
+        for (int i = 0; i < WI; ++i) {
+            const uint8_t* base;
+            int n;
+            if (SWIGLU) {
+                base = wrow[i] < BN / 2 ? p.b : p.b2;
+                n = n0 + (wrow[i] < BN / 2 ? wrow[i] : wrow[i] - BN / 2);
+            } else {
+                base = p.b;
+                n = n0 + wrow[i];
             }
+            n = n < p.N ? n : p.N - 1;
+            wptr[i] = base + ((int64_t)t.expert * p.b_se + (int64_t)n * p.b_sn) * ESIZE + wsw[i];
+        }
+    };
+    auto issue = [&](int kt, int slot_i) {
+        const uint32_t sbase = lds_base + slot_i * TL::STAGE_BYTES;
+        const int64_t koff = (int64_t)kt * 64;
 #pragma unroll
-            for (int fm = 0; fm < FM; ++fm) {
-                uint32_t packed[4];
+        for (int i = 0; i < XI; ++i) dma16(xptr[i] + koff, sbase + (i * NW + wave) * 1024);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float y = acc[fn][fm][4 * g + j];
-                    float y2 = SWIGLU ? acc[fn + FN / 2][fm][4 * g + j] : 0.0f;
-                    if (FP8) {
-                        // (acc / (sa * sw)) rounded to bf16, then the bias added in bf16
-                        y = round_bf16(y * (rsa[fm] * rsw[j]));
-                        if (p.bias) y = round_bf16(y + bv[j]);
-                        if (SWIGLU) {
-                            y2 = round_bf16(y2 * (rsa[fm] * rsw2[j]));
-                            if (p.bias2) y2 = round_bf16(y2 + bv2[j]);
-                        }
-                    } else {
-                        y = round_bf16(y + bv[j]);
-                        if (SWIGLU) y2 = round_bf16(y2 + bv2[j]);
-                    }
-                    if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
-                    if (SWIGLU) y = round_bf16(fast_silu_f32(y)) * y2;
-                    packed[j] = f32_to_bf16_bits(y);
+        for (int i = 0; i < WI; ++i) dma16(wptr[i] + koff, sbase + BM * 64 + (i * NW + wave) * 1024);
+    };
+
+    int wfrag_row[FN], xfrag_row[FM];
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+        int r;
+        if (SWIGLU) r = (fn < FN / 2 ? 0 : BN / 2) + wn * (TN / 2) + (fn % (FN / 2)) * 32;
+        else r = wn * TN + fn * 32;
+        wfrag_row[fn] = r + (lane & 31);
+    }
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) xfrag_row[fm] = wm * TM + fm * 32 + (lane & 31);
+
+    const int KT = p.K / BK;
+    int64_t logical = xcd_begin + slot;
+    if (logical >= xcd_end) return;
+    const int my_tiles = (int)((xcd_end - logical + nslots - 1) / nslots);
+    const int total_items = my_tiles * KT;
+
+    // The block's work is one flat stream of K-slices ("items"): KT per tile, tile after
+    // tile.  Item i lives in ring slot i % STAGES.  The issue side runs STAGES-1 items ahead
+    // of the compute side and crosses tile boundaries on its own; it only needs the row
+    // pointers of the tile it is in, the compute side only the TileInfo for the epilogue.
+    TileInfo cur = locate(logical);         // tile being computed
+    TileInfo nxt = cur;                     // tile after it (located one tile ahead)
+    int64_t ilogical = logical;
+    int ikt = 0;                            // next K-slice to issue inside the issue tile
+    int issued = 0;                         // items issued so far
+    int64_t ridx_next[XI];
+    {
+        int64_t r0[XI];
+        fetch_rows(cur, r0);
+        make_ptrs(cur, r0);
+    }
+    auto issue_one = [&]() {
+        if (issued >= total_items) return;
+        if (ikt == KT) {                    // the issue side enters the next tile
+            make_ptrs(nxt, ridx_next);
+            ikt = 0;
+        }
+        issue(ikt, issued % STAGES);
+        ++ikt;
+        ++issued;
+    };
+    auto prefetch_next = [&]() {            // once per tile, early: locate the next tile and
+        ilogical += nslots;                 // start fetching its source-row indices
+        if (ilogical < xcd_end) {
+            nxt = locate(ilogical);
+            fetch_rows(nxt, ridx_next);
+        }
+    };
+    prefetch_next();
+    for (int j = 0; j < STAGES - 1; ++j) issue_one();
+
+    // vmcnt bookkeeping.  Loads return in order, so "at most n*L operations outstanding"
+    // means every slice but the n youngest has landed; stores or other loads in the queue
+    // only make the wait longer, never shorter.
+    int landed = -1;                        // items <= landed are complete for this wave
+    int c = 0;                              // item being computed
+    for (int tile_i = 0; tile_i < my_tiles; ++tile_i) {
+        f32x16 acc[FN][FM];
+#pragma unroll
+        for (int i = 0; i < FN; ++i)
+#pragma unroll
+            for (int j = 0; j < FM; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        if (tile_i > 0) prefetch_next();
+
+        for (int kt = 0; kt < KT; ++kt, ++c) {
+            if (c > landed) {
+                const int younger = issued - 1 - c;
+                if (younger >= 2) wait_vmcnt<2 * L>();
+                else if (younger == 1) wait_vmcnt<L>();
+                else wait_vmcnt<0>();
+            }
+            // after this barrier every wave's share of item c is visible and every wave has
+            // finished reading item c-1, whose slot the next issue overwrites
+            __syncthreads();
+            issue_one();
+            const uint8_t* sx = smem + (c % STAGES) * TL::STAGE_BYTES;
+            const uint8_t* sw = sx + BM * 64;
+            if (!FP8) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const int chunk = 2 * s + khalf;
+                    bf16x8 wf[FN], xf[FM];
+#pragma unroll
+                    for (int fn = 0; fn < FN; ++fn)
+                        wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
+#pragma unroll
+                    for (int fm = 0; fm < FM; ++fm)
+                        xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
+#pragma unroll
+                    for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+                        for (int fm = 0; fm < FM; ++fm)
+                            acc[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0);
                 }
-                if (!row_ok[fm]) continue;
-                if (p.vec_store && nb + 3 < p.N) {
-                    u32x2 o;
-                    o[0] = packed[0] | (packed[1] << 16);
-                    o[1] = packed[2] | (packed[3] << 16);
-                    *reinterpret_cast<u32x2*>(orow[fm] + nb) = o;
-                } else {
+            } else {
+                const int chunk = 2 * khalf;
+                i32x8 wf[FN], xf[FM];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (nb + j < p.N) orow[fm][nb + j] = (uint16_t)packed[j];
+                for (int fn = 0; fn < FN; ++fn) {
+                    const u32x4 lo = *reinterpret_cast<const u32x4*>(sw + lds_off64(wfrag_row[fn], chunk));
+                    const u32x4 hi = *reinterpret_cast<const u32x4*>(sw + lds_off64(wfrag_row[fn], chunk + 1));
+                    wf[fn] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
                 }
+#pragma unroll
+                for (int fm = 0; fm < FM; ++fm) {
+                    const u32x4 lo = *reinterpret_cast<const u32x4*>(sx + lds_off64(xfrag_row[fm], chunk));
+                    const u32x4 hi = *reinterpret_cast<const u32x4*>(sx + lds_off64(xfrag_row[fm], chunk + 1));
+                    xf[fm] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                }
+#pragma unroll
+                for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+                    for (int fm = 0; fm < FM; ++fm)
+                        acc[fn][fm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0, 0, 0, 0);
             }
         }
+        // All but the youngest issued slice have landed after this wait, so the first slices
+        // of the next tile need no vmcnt wait and the epilogue's stores drain behind them.
+        wait_vmcnt<L>();
+        landed = issued - 2;
+        const TileInfo done = cur;
+        cur = nxt;      // valid when another tile follows (nxt was located at this tile's start)
+
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
+                                                done.rows_valid, wm, wn, lane);
     }
 }
 
+
 // ------------------------------------------------------------------- host side
-typedef TileCfg<256, 256, 2, 4> TileBig;     // 8 waves, wave tile 128 x 64
-typedef TileCfg<64, 256, 1, 4> TileSmall;    // 4 waves, wave tile 64 x 64
+typedef TileCfg<256, 256, 2, 4> TileBig;        // 8 waves, wave tile 128 x 64
+typedef TileCfg<64, 256, 1, 4> TileSmall;       // 4 waves, wave tile 64 x 64
+typedef RingCfg<256, 256, 2, 4, 4> TileRing;    // 8 waves, wave tile 128 x 64, 4-slot ring
+
+enum GemmKernelSel { kSelRing = 0, kSelStagedBig = 1, kSelStagedSmall = 2, kSelGeneric = 3 };
+
+template <typename Kern>
+int reserve_lds(Kern kern, int bytes, bool& done) {
+    if (done) return FMOE_OK;
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (err != hipSuccess)
+        return fail(FMOE_ERR_LAUNCH, "fmoe_grouped_gemm: cannot reserve %d B of LDS: %s", bytes,
+                    hipGetErrorString(err));
+    done = true;
+    return FMOE_OK;
+}
 
 template <typename TL, bool FP8, int EPI, bool FAST, bool A_SILU>
 int launch_gemm(GemmParams p, hipStream_t stream) {
@@ -424,14 +801,7 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
     auto kern = grouped_gemm_kernel<TL, FP8, EPI, FAST, A_SILU>;
     static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES);
-        if (err != hipSuccess)
-            return fail(FMOE_ERR_LAUNCH, "fmoe_grouped_gemm: cannot reserve %d B of LDS: %s", TL::LDS_BYTES,
-                        hipGetErrorString(err));
-        attr_done = true;
-    }
+    if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
     const int64_t max_m_tiles = p.total_rows / TL::BM + p.E;
     const int64_t max_tiles = max_m_tiles * p.n_tiles;
     const int64_t grid = (max_tiles + kNumXcd - 1) / kNumXcd * kNumXcd;
@@ -440,15 +810,38 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
     return check_launch("fmoe_grouped_gemm");
 }
 
+int compute_units();   // CUs of the current device (gemm_api.hip)
+
+template <bool FP8, int EPI>
+int launch_ring(GemmParams p, hipStream_t stream) {
+    typedef TileRing TL;
+    constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
+    p.n_tiles = (p.N + bn_out - 1) / bn_out;
+    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI>;
+    static bool attr_done = false;
+    if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
+    // persistent: one block per CU (the LDS footprint admits no second one), a multiple of
+    // the XCD count so that every XCD owns the same number of blocks
+    int grid = compute_units() / kNumXcd * kNumXcd;
+    if (grid < kNumXcd) grid = kNumXcd;
+    kern<<<(unsigned)grid, TL::NT, TL::LDS_BYTES, stream>>>(p);
+    return check_launch("fmoe_grouped_gemm");
+}
+
 template <bool FP8, int EPI, bool A_SILU>
-int dispatch_tile(const GemmParams& p, bool fast, bool big, hipStream_t stream) {
-    if (!fast) return launch_gemm<TileSmall, FP8, EPI, false, A_SILU>(p, stream);
-    if (big) return launch_gemm<TileBig, FP8, EPI, true, A_SILU>(p, stream);
-    return launch_gemm<TileSmall, FP8, EPI, true, A_SILU>(p, stream);
+int dispatch_tile(const GemmParams& p, int sel, hipStream_t stream) {
+    switch (sel) {
+        case kSelRing:
+            if constexpr (!A_SILU) return launch_ring<FP8, EPI>(p, stream);
+            else return launch_gemm<TileBig, FP8, EPI, true, A_SILU>(p, stream);
+        case kSelStagedBig: return launch_gemm<TileBig, FP8, EPI, true, A_SILU>(p, stream);
+        case kSelStagedSmall: return launch_gemm<TileSmall, FP8, EPI, true, A_SILU>(p, stream);
+        default: return launch_gemm<TileSmall, FP8, EPI, false, A_SILU>(p, stream);
+    }
 }
 
 // Entry points of the two translation units.
-int run_gemm_bf16(GemmParams& p, int epilogue, bool a_silu, bool fast, bool big, hipStream_t stream);
-int run_gemm_fp8(GemmParams& p, int epilogue, bool fast, bool big, hipStream_t stream);
+int run_gemm_bf16(GemmParams& p, int epilogue, bool a_silu, int sel, hipStream_t stream);
+int run_gemm_fp8(GemmParams& p, int epilogue, int sel, hipStream_t stream);
 
 }  // namespace fmoe
