@@ -28,6 +28,12 @@ if ROOT not in sys.path:
 
 PEAK = {"bf16": 2500.0, "fp8": 5000.0}   # dense MFMA TFLOP/s, MI355X
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per GEMM1 launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
+# profiles/ (KiB per dispatch, scaled by the copy-kernel factors 2.0 and 1.0 stated there).
+MEASURED_TRAFFIC_BYTES = {
+    "c3_bf16": int((1.6528e6 * 2.0 + 3.8075e5 * 1.0) * 1024),
+    "c4_fp8": int((8.7197e5 * 2.0 + 3.7133e5 * 1.0) * 1024),
+}
 
 WORKLOADS = {
     # name: (T, E, K, D, H, O, kind, dtype, routing)
@@ -280,6 +286,8 @@ def main():
     ap.add_argument("--tokens", type=int, default=None, help="override the token count (C5 sweep)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary fp8 / bf16 workload")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 512 MiB device copy, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU with all experts local; expert parallelism is out of "
@@ -306,7 +314,8 @@ def main():
         "roofline": {"bound": "mfma", "kernel": "grouped_gemm (gemm1: gather + GEMM + " +
                      ("SwiGLU" if w["kind"] == "swiglu" else "SiLU") + " epilogue)",
                      "achieved": g1["tflops"], "peak": PEAK[dt], "unit": "TFLOP/s",
-                     "frac": round(g1["tflops"] / PEAK[dt], 4), "traffic": None},
+                     "frac": round(g1["tflops"] / PEAK[dt], 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if not args.tokens else None},
     }
     if not args.no_extra:
         other = {"c3_bf16": "c4_fp8", "c4_fp8": "c3_bf16"}.get(args.workload)
@@ -315,6 +324,13 @@ def main():
             line["extra"] = {other: {"value": round(fl2 / ms2 / 1e9, 2), "unit": "TFLOP/s",
                                      "ms_per_step": round(ms2, 4), "tokens_per_s": round(w2["T"] / ms2 * 1e3, 1),
                                      "kernels": k2}}
+    if args.calibrate_copy:      # a kernel of known traffic: 512 MiB read + 512 MiB written
+        src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        line["calibration"] = {"kernel": "torch Tensor.copy_ of 536870912 bytes (uint8)", "launches": 3}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w)
     print(json.dumps(line))
