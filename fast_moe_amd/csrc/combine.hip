@@ -61,56 +61,101 @@ __device__ __forceinline__ float gate_of(const GateView& g, int64_t r, bool& ok)
 
 // TV value dtype, TG gate dtype, ROUND_BF16: the product is rounded to bf16
 // (both operands bf16); HAS_GATE false = plain segmented sum.
-// VECTOR: 16-byte loads, one wave covers 64*kVec columns of one token.
-template <typename TV, typename TG, typename TO, bool HAS_GATE, bool ROUND_BF16, bool VECTOR>
+// VECTOR: 16-byte loads; one wave covers CPW * 64 * kVec consecutive columns of one token.
+// The K source rows and gates of the token are fetched by lanes 0..K-1 in three parallel
+// rounds (reverse_index -> gates_index -> gate) and handed out with readlane; rows are
+// loaded in batches of JB with all loads of a batch in flight, then added in order.
+template <typename TV, typename TG, typename TO, bool HAS_GATE, bool ROUND_BF16, bool VECTOR, int CPW>
 __global__ __launch_bounds__(256) void combine_kernel(const TV* __restrict__ value, int64_t T, int K,
                                                       int64_t D, int64_t stride_row,
                                                       const int64_t* __restrict__ reverse_index,
                                                       GateView gate, TO* __restrict__ out,
-                                                      int chunks_per_token) {
+                                                      int groups_per_token) {
     constexpr int VEC = VECTOR ? Elem<TV>::kVec : 1;
+    constexpr int JB = 8;
     const int lane = lane_id();
     const int64_t wave = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
-    const int64_t t = wave / chunks_per_token;
-    const int chunk = (int)(wave - t * chunks_per_token);
+    const int64_t t = wave / groups_per_token;
+    const int group = (int)(wave - t * groups_per_token);
     if (t >= T) return;
-    const int64_t col = ((int64_t)chunk * kWave + lane) * VEC;
-    const bool active = col < D;
     const int64_t R = T * K;
-    float acc[VEC];
+
+    // lanes 0..K-1 (K <= 64 per pass) own one source row each
+    float acc[CPW][VEC];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) acc[i] = 0.0f;
-#pragma unroll 4
-    for (int j = 0; j < K; ++j) {
-        const int64_t r = reverse_index[t * K + j];
-        if ((uint64_t)r >= (uint64_t)R) continue;       // malformed index: contributes nothing
-        float w = 1.0f;
-        if (HAS_GATE) {
-            bool ok;
-            w = gate_of<TG>(gate, r, ok);
-            if (!ok) continue;
-        }
-        if (!active) continue;
-        float f[VEC];
-        if (VECTOR) {
-            const u32x4 raw = *reinterpret_cast<const u32x4*>(value + r * stride_row + col);
-            Elem<TV>::unpack(raw, f);
-        } else {
-            f[0] = Elem<TV>::load(value + r * stride_row + col);
-        }
+    for (int c = 0; c < CPW; ++c)
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) {
-            float p = HAS_GATE ? f[i] * w : f[i];
-            if (HAS_GATE && ROUND_BF16) p = round_bf16(p);
-            acc[i] = acc[i] + p;
+        for (int i = 0; i < VEC; ++i) acc[c][i] = 0.0f;
+    int64_t col[CPW];
+    bool active[CPW];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+        col[c] = (((int64_t)group * CPW + c) * kWave + lane) * VEC;
+        active[c] = col[c] < D;
+    }
+
+    for (int k0 = 0; k0 < K; k0 += kWave) {
+        const int kn = K - k0 < kWave ? K - k0 : kWave;
+        int64_t my_r = -1;
+        float my_w = 1.0f;
+        if (lane < kn) {
+            my_r = reverse_index[t * K + k0 + lane];
+            if ((uint64_t)my_r >= (uint64_t)R) my_r = -1;        // malformed index: contributes nothing
+            if (HAS_GATE && my_r >= 0) {
+                bool ok;
+                my_w = gate_of<TG>(gate, my_r, ok);
+                if (!ok) my_r = -1;
+            }
+        }
+        for (int j0 = 0; j0 < kn; j0 += JB) {
+            u32x4 raw[JB][CPW];
+            float sv[JB][CPW];
+            int64_t rj[JB];
+            float wj[JB];
+#pragma unroll
+            for (int jj = 0; jj < JB; ++jj) {
+                const int j = j0 + jj < kn ? j0 + jj : kn - 1;
+                rj[jj] = wave_bcast(my_r, j);
+                wj[jj] = wave_bcast(my_w, j);
+                if (j0 + jj >= kn) rj[jj] = -1;
+#pragma unroll
+                for (int c = 0; c < CPW; ++c) {
+                    raw[jj][c] = u32x4{0, 0, 0, 0};
+                    sv[jj][c] = 0.0f;
+                    if (rj[jj] >= 0 && active[c]) {
+                        const TV* src = value + rj[jj] * stride_row + col[c];
+                        if (VECTOR) raw[jj][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
+                        else sv[jj][c] = Elem<TV>::load(src);
+                    }
+                }
+            }
+#pragma unroll
+            for (int jj = 0; jj < JB; ++jj) {
+                if (rj[jj] < 0) continue;
+#pragma unroll
+                for (int c = 0; c < CPW; ++c) {
+                    float f[VEC];
+                    if (VECTOR) Elem<TV>::unpack(raw[jj][c], f);
+                    else f[0] = sv[jj][c];
+#pragma unroll
+                    for (int i = 0; i < VEC; ++i) {
+                        float p = HAS_GATE ? f[i] * wj[jj] : f[i];
+                        if (HAS_GATE && ROUND_BF16) p = round_bf16(p);
+                        acc[c][i] = acc[c][i] + p;
+                    }
+                }
+            }
         }
     }
-    if (!active) return;
-    if (VECTOR && sizeof(TO) == sizeof(TV)) {
-        *reinterpret_cast<u32x4*>(out + t * D + col) = Elem<TO>::pack(acc);
-    } else {
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) Elem<TO>::store(out + t * D + col + i, acc[i]);
+    for (int c = 0; c < CPW; ++c) {
+        if (!active[c]) continue;
+        if (VECTOR && sizeof(TO) == sizeof(TV)) {
+            *reinterpret_cast<u32x4*>(out + t * D + col[c]) = Elem<TO>::pack(acc[c]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) Elem<TO>::store(out + t * D + col[c] + i, acc[c][i]);
+        }
     }
 }
 
@@ -119,16 +164,19 @@ void launch(const void* value, int64_t T, int K, int64_t D, int64_t stride_row,
             const int64_t* reverse_index, const GateView& gate, void* out, hipStream_t stream) {
     constexpr int vec = Elem<TV>::kVec;
     const bool vector = (D % vec) == 0 && (stride_row % vec) == 0 && aligned16(value) && aligned16(out);
-    const int per_wave = kWave * (vector ? vec : 1);
-    const int chunks = (int)((D + per_wave - 1) / per_wave);
-    const int64_t waves = T * chunks;
+    const int per_chunk = kWave * (vector ? vec : 1);
+    const int chunks = (int)((D + per_chunk - 1) / per_chunk);
+    const bool wide = vector && chunks >= 2;                 // two 16-byte chunks per lane
+    const int groups = wide ? (chunks + 1) / 2 : chunks;
+    const int64_t waves = T * groups;
     const unsigned blocks = (unsigned)((waves + 3) / 4);
-    if (vector)
-        combine_kernel<TV, TG, TO, HAS_GATE, ROUND_BF16, true><<<blocks, 256, 0, stream>>>(
-            (const TV*)value, T, K, D, stride_row, reverse_index, gate, (TO*)out, chunks);
-    else
-        combine_kernel<TV, TG, TO, HAS_GATE, ROUND_BF16, false><<<blocks, 256, 0, stream>>>(
-            (const TV*)value, T, K, D, stride_row, reverse_index, gate, (TO*)out, chunks);
+#define FMOE_COMBINE(VECTOR, CPW)                                                                  \
+    combine_kernel<TV, TG, TO, HAS_GATE, ROUND_BF16, VECTOR, CPW><<<blocks, 256, 0, stream>>>(        \
+        (const TV*)value, T, K, D, stride_row, reverse_index, gate, (TO*)out, groups)
+    if (wide) FMOE_COMBINE(true, 2);
+    else if (vector) FMOE_COMBINE(true, 1);
+    else FMOE_COMBINE(false, 1);
+#undef FMOE_COMBINE
 }
 
 }  // namespace

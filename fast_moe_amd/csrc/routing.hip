@@ -7,17 +7,17 @@
 // Pipeline (4 launches on one stream, no host synchronisation):
 //   1. topk_kernel     rank-by-counting selection, one token per LPT lanes
 //   2. hist_kernel     one wave per chunk of tokens: LDS histogram -> chunk_hist[c][e]
-//   3. scan_kernel     one block: exclusive scan of chunk_hist over chunks (in
-//                      place), lengths[e], offsets[e] (wave scan over experts)
-//   4. scatter_kernel  one wave per chunk: wave-level match/rank gives each
-//                      position its slot inside its expert segment
+//   3. scan_kernel     one block per expert: exclusive scan of chunk_hist over the
+//                      chunks (in place, wave scans), lengths[e]
+//   4. scatter_kernel  one wave per chunk: offsets = wave scan of lengths, then a
+//                      wave-level match/rank gives each position its slot inside
+//                      its expert segment
 #include "common.h"
 
 namespace fmoe {
 namespace {
 
 constexpr int kMaxChunks = 512;
-constexpr int kScanThreads = 1024;
 constexpr uint16_t kBadExpert = 0xFFFF;
 
 struct RoutePlan {
@@ -93,9 +93,12 @@ __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores,
     for (int v = 0; v < VPL; ++v) rank[v] = 0;
 #pragma unroll
     for (int u = 0; u < VPL; ++u) {
-#pragma unroll 8
+#pragma unroll
         for (int i = 0; i < LPT; ++i) {
-            const float other = __shfl(my[u], grp * LPT + i, kWave);
+            // a full wave per token: the broadcast lane is a compile-time constant (v_readlane)
+            const float other = LPT == kWave
+                                    ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my[u]), i))
+                                    : __shfl(my[u], grp * LPT + i, kWave);
             const int oe = u * LPT + i;
 #pragma unroll
             for (int v = 0; v < VPL; ++v) {
@@ -163,58 +166,25 @@ __global__ __launch_bounds__(kWave) void hist_kernel(const uint16_t* __restrict_
     for (int e = threadIdx.x; e < E; e += kWave) chunk_hist[(int64_t)c * E + e] = s_cnt[e];
 }
 
-// Single block.  Threads form [SEG][EW] (EW = power of two >= E): thread (s, e)
-// owns chunks [s*cps, (s+1)*cps) of expert e.
-__global__ __launch_bounds__(kScanThreads) void scan_kernel(int32_t* __restrict__ chunk_hist,
-                                                            int num_chunks, int E, int EW,
-                                                            int64_t* __restrict__ lengths,
-                                                            int64_t* __restrict__ offsets) {
-    extern __shared__ int32_t s_buf[];   // [SEG][EW] partials, then [E] totals
-    const int SEG = kScanThreads / EW;
-    const int e = threadIdx.x % EW;
-    const int s = threadIdx.x / EW;
-    const int cps = (num_chunks + SEG - 1) / SEG;
-    const int c0 = s * cps;
-    int c1 = c0 + cps;
-    if (c1 > num_chunks) c1 = num_chunks;
-    int32_t part = 0;
-    if (e < E)
-        for (int c = c0; c < c1; ++c) part += chunk_hist[(int64_t)c * E + e];
-    s_buf[s * EW + e] = part;
+// One block per expert: exclusive scan of that expert's counts over the chunks (in place)
+// and its total.  256 threads, two chunks per thread (num_chunks <= 512).
+__global__ __launch_bounds__(256) void scan_kernel(int32_t* __restrict__ chunk_hist, int num_chunks, int E,
+                                                   int64_t* __restrict__ lengths) {
+    __shared__ int32_t s_wave[4];
+    const int e = blockIdx.x;
+    const int c0 = threadIdx.x * 2, c1 = c0 + 1;
+    const int32_t v0 = c0 < num_chunks ? chunk_hist[(int64_t)c0 * E + e] : 0;
+    const int32_t v1 = c1 < num_chunks ? chunk_hist[(int64_t)c1 * E + e] : 0;
+    const int inc = wave_inclusive_scan((int)(v0 + v1));
+    const int wave = threadIdx.x / kWave;
+    if (lane_id() == kWave - 1) s_wave[wave] = inc;
     __syncthreads();
-    int32_t base = 0, total = 0;
-    for (int q = 0; q < SEG; ++q) {
-        const int32_t v = s_buf[q * EW + e];
-        if (q < s) base += v;
-        total += v;
-    }
-    if (e < E) {
-        int32_t run = base;
-        for (int c = c0; c < c1; ++c) {
-            const int64_t i = (int64_t)c * E + e;
-            const int32_t v = chunk_hist[i];
-            chunk_hist[i] = run;
-            run += v;
-        }
-    }
-    __syncthreads();
-    int32_t* s_tot = s_buf;
-    if (s == 0 && e < E) {
-        s_tot[e] = total;
-        lengths[e] = total;
-    }
-    __syncthreads();
-    if (threadIdx.x < kWave) {
-        long long run = 0;
-        if (threadIdx.x == 0) offsets[0] = 0;
-        for (int e0 = 0; e0 < E; e0 += kWave) {
-            const int ee = e0 + threadIdx.x;
-            const long long v = ee < E ? (long long)s_tot[ee] : 0;
-            const long long inc = wave_inclusive_scan(v);
-            if (ee < E) offsets[ee + 1] = run + inc;
-            run += wave_bcast(inc, kWave - 1);
-        }
-    }
+    int base = 0;
+    for (int w = 0; w < wave; ++w) base += s_wave[w];
+    const int excl = base + inc - (v0 + v1);
+    if (c0 < num_chunks) chunk_hist[(int64_t)c0 * E + e] = excl;
+    if (c1 < num_chunks) chunk_hist[(int64_t)c1 * E + e] = excl + v0;
+    if (threadIdx.x == 255) lengths[e] = base + inc;
 }
 
 // One wave per chunk.  Each iteration takes TPI = 64/K whole tokens, lane i <->
@@ -224,15 +194,28 @@ __global__ __launch_bounds__(kWave) void scatter_kernel(const uint16_t* __restri
                                                         int64_t num_tokens, int64_t tokens_per_chunk,
                                                         int E, int K, int ebits,
                                                         const int32_t* __restrict__ chunk_base,
-                                                        const int64_t* __restrict__ offsets,
+                                                        const int64_t* __restrict__ lengths,
+                                                        int64_t* __restrict__ offsets,
                                                         int64_t* __restrict__ gate_index,
                                                         int64_t* __restrict__ token_index,
                                                         int64_t* __restrict__ reverse_index) {
     extern __shared__ int32_t s_next[];
     const int c = blockIdx.x;
     const int lane = threadIdx.x;
-    for (int e = lane; e < E; e += kWave)
-        s_next[e] = (int32_t)offsets[e] + chunk_base[(int64_t)c * E + e];
+    {   // exclusive prefix of lengths over the experts = offsets (wave scan); chunk 0 publishes it
+        long long run = 0;
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int e = e0 + lane;
+            const long long v = e < E ? (long long)lengths[e] : 0;
+            const long long inc = wave_inclusive_scan(v);
+            if (e < E) {
+                s_next[e] = (int32_t)(run + inc - v) + chunk_base[(int64_t)c * E + e];
+                if (c == 0) offsets[e] = run + inc - v;
+            }
+            run += wave_bcast(inc, kWave - 1);
+        }
+        if (c == 0 && lane == 0) offsets[E] = run;
+    }
     __syncthreads();
     const int tpi = kWave / K;
     const int64_t t_begin = (int64_t)c * tokens_per_chunk;
@@ -287,12 +270,9 @@ int launch_sort(const uint16_t* compact, int32_t* chunk_hist, const RoutePlan& p
     const int64_t total_pos = T * K;
     hist_kernel<<<plan.num_chunks, kWave, E * sizeof(int32_t), stream>>>(
         compact, total_pos, plan.tokens_per_chunk * K, E, chunk_hist);
-    int EW = 1;
-    while (EW < E) EW <<= 1;
-    scan_kernel<<<1, kScanThreads, kScanThreads * sizeof(int32_t), stream>>>(
-        chunk_hist, plan.num_chunks, E, EW, lengths, offsets);
+    scan_kernel<<<E, 256, 0, stream>>>(chunk_hist, plan.num_chunks, E, lengths);
     scatter_kernel<<<plan.num_chunks, kWave, E * sizeof(int32_t), stream>>>(
-        compact, T, plan.tokens_per_chunk, E, K, ceil_log2(E), chunk_hist, offsets, gate_index,
+        compact, T, plan.tokens_per_chunk, E, K, ceil_log2(E), chunk_hist, lengths, offsets, gate_index,
         token_index, reverse_index);
     return check_launch("routing sort");
 }
