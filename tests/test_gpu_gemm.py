@@ -268,3 +268,118 @@ def test_forward_only_and_dtype_errors():
     with pytest.raises(NotImplementedError):
         with torch.no_grad():
             moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x.float(), w.float(), None)
+
+
+# ------------------------------------------------------------- ring-kernel specifics
+@pytest.mark.parametrize("L,E,K,Din,Dout,epi", [
+    (4096, 8, 2, 96, 256, "plain"),        # three K-slices only: the ring never fills
+    (4096, 8, 2, 1024, 264, "plain"),      # N = 264: last column tile 8 wide
+    (9000, 3, 1, 512, 512, "plain"),       # fewer tiles than CUs, K_top = 1 (index_shift 0)
+    (6144, 24, 3, 256, 384, "swiglu"),     # top-3: index division, not a shift
+    (20000, 200, 2, 128, 128, "swiglu"),   # many experts, about 200 rows each
+    (3000, 2, 2, 2048, 128, "swiglu"),     # long K, one column tile
+])
+def test_ring_kernel_shapes(L, E, K, Din, Dout, epi):
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=L + E)
+    x = randn((L, Din), 1)
+    w = weights(E, Din, Dout, 2, False, scale=Din ** -0.5)
+    b = randn((E, Dout), 3)
+    if epi == "plain":
+        ref = o_moe.index_select_jagged_bmm(r["offsets"], r["index"], x.float(), w.float(), b.float())
+        with torch.no_grad():
+            out = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b))
+        assert_bf16_close(out, ref, rtol=1e-2, atol=1e-2, what=f"ring plain {L},{E},{K},{Din},{Dout}")
+    else:
+        wp = weights(E, Din, Dout, 5, False, scale=Din ** -0.5)
+        ref = o_moe.index_select_jagged_bmm_swiglu(r["offsets"], r["index"], x.float(), w.float(), b.float(),
+                                                   wp.float(), None)
+        with torch.no_grad():
+            out = moe.index_select_jagged_bmm_swiglu(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b),
+                                                     dev(wp), None)
+        assert_bf16_close(out, ref, rtol=1.6e-2, atol=1e-2, what=f"ring swiglu {L},{E},{K},{Din},{Dout}")
+
+
+def test_ring_kernel_is_deterministic_and_ignores_garbage_offsets():
+    """Two launches give identical bits; offsets outside [0, R] are clamped instead of followed."""
+    from fast_moe_amd.kernels.hip import ops
+    L, E, K, D, N = 8192, 16, 2, 256, 256
+    r = make_routing(L, E, K, seed=5)
+    x, w = dev(randn((L, D), 1)), dev(weights(E, D, N, 2, False, scale=D ** -0.5))
+    a = ops.grouped_gemm(dev(r["offsets"]), x, w, total_rows=L * K, row_index=dev(r["gate_index"]), index_div=K)
+    b = ops.grouped_gemm(dev(r["offsets"]), x, w, total_rows=L * K, row_index=dev(r["gate_index"]), index_div=K)
+    assert torch.equal(a, b)
+    bad = r["offsets"].clone()
+    bad[-1] = 10 ** 12
+    bad[3] = -7
+    out = ops.grouped_gemm(dev(bad), x, w, total_rows=L * K, row_index=dev(r["gate_index"]), index_div=K)
+    torch.cuda.synchronize()
+    assert out.shape == a.shape
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_full_size_c3_c4_sampled_rows(fp8):
+    """BASELINE sizes (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed, empty experts): the
+    whole SwiGLU GEMM runs on the GPU, a sample of its rows is checked against the oracle, and
+    size-independent properties hold (rows of empty experts absent, duplicate tokens give equal rows)."""
+    from fast_moe_amd.kernels import moe_fp8
+    from fast_moe_amd.kernels.hip import ops
+    T, E, K, D, H = 16384, 64, 8, 2048, 1408
+    topk = skewed_topk(T, E, K, seed=11)
+    meta = o_routing.routing_metadata(topk.numpy(), E)
+    assert (meta["lengths"] == 0).sum() >= 2
+    offsets = torch.from_numpy(meta["offsets"])
+    gate_index = torch.from_numpy(meta["gate_index"])
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(T, D, generator=g).to(BF16)
+    x[5] = x[4]                                            # two identical tokens
+    if fp8:
+        x[::100] *= 100
+    wg = (torch.randn(E, H, D, generator=g) * D ** -0.5).to(BF16).permute(0, 2, 1)
+    wu = (torch.randn(E, H, D, generator=g) * D ** -0.5).to(BF16).permute(0, 2, 1)
+    with torch.no_grad():
+        if fp8:
+            qg, sg = moe_fp8.quantize_expert_weights(dev(wg))
+            qu, su = moe_fp8.quantize_expert_weights(dev(wu))
+            qx, sx = ops.quant_rows_fp8(dev(x))
+            out = ops.grouped_gemm(dev(offsets), qx, qg, total_rows=T * K, row_index=dev(gate_index), index_div=K,
+                                   b2=qu, epilogue=2, a_scale=sx, b_scale=sg, b2_scale=su)
+        else:
+            out = ops.grouped_gemm(dev(offsets), dev(x), dev(wg), total_rows=T * K, row_index=dev(gate_index),
+                                   index_div=K, b2=dev(wu), epilogue=2)
+    out = out.cpu()
+    assert bool(torch.isfinite(out).all())
+    rows = torch.randperm(T * K, generator=g)[:192]
+    experts = torch.searchsorted(offsets[1:], rows, right=True)
+    tok = gate_index[rows] // K
+    for i in range(rows.numel()):
+        e, t = int(experts[i]), int(tok[i])
+        if fp8:
+            one = torch.tensor([0, 1])
+            eo = torch.zeros(2, dtype=torch.int64)
+            eo[1] = 1
+            # the oracle's fp8 path on a single row / single expert
+            from oracle import moe_fp8 as o8
+            qa, sa = o8.rowwise_quant_fp8(x[t:t + 1])
+            qwg, swg = o8.rowwise_quant_fp8(wg[e:e + 1].permute(0, 2, 1))
+            qwu, swu = o8.rowwise_quant_fp8(wu[e:e + 1].permute(0, 2, 1))
+            gg = o8.fp8_linear_per_expert([o8.dequant(qa)], [sa], o8.dequant(qwg), swg, None, BF16)[0]
+            uu = o8.fp8_linear_per_expert([o8.dequant(qa)], [sa], o8.dequant(qwu), swu, None, BF16)[0]
+            ref = (torch.nn.functional.silu(gg) * uu)[0]
+            tol = 3e-2
+        else:
+            xr = x[t].float()
+            ref = torch.nn.functional.silu(xr @ wg[e].float()) * (xr @ wu[e].float())
+            tol = 1.6e-2
+        err = (out[rows[i]].float() - ref.float()).abs()
+        scale = ref.float().abs().max().item()
+        assert bool((err <= tol * ref.float().abs() + tol * scale * 0.5 + 1e-3).all()), (int(rows[i]), err.max())
+    # identical tokens routed to the same expert give identical rows
+    pos = {}
+    for tkn in (4, 5):
+        for j in range(K):
+            pos[(tkn, int(topk[tkn, j]))] = int(torch.from_numpy(meta["reverse_index"])[tkn][
+                sorted(range(K), key=lambda q: int(topk[tkn, q])).index(j)])
+    common = set(int(e) for e in topk[4]) & set(int(e) for e in topk[5])
+    for e in common:
+        assert torch.equal(out[pos[(4, e)]], out[pos[(5, e)]])
