@@ -60,10 +60,52 @@ __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __re
     }
 }
 
+// 64 x 64 tile transpose through LDS; reads and writes are both row-contiguous
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst,
+                                                        int64_t rows, int64_t cols, int64_t sb, int64_t sr) {
+    __shared__ T tile[64][64 + 2];
+    const int64_t b = blockIdx.z;
+    const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    const T* s = src + b * sb;
+    T* d = dst + b * rows * cols;
+    for (int i = ty; i < 64; i += 4) {
+        const int64_t r = r0 + i, c = c0 + tx;
+        if (r < rows && c < cols) tile[i][tx] = s[r * sr + c];
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const int64_t c = c0 + i, r = r0 + tx;
+        if (r < rows && c < cols) d[c * rows + r] = tile[tx][i];
+    }
+}
+
 }  // namespace
 }  // namespace fmoe
 
 using namespace fmoe;
+
+extern "C" int fmoe_transpose_last2(const void* src, void* dst, int elem_size, int64_t batch, int64_t rows,
+                                    int64_t cols, int64_t src_stride_b, int64_t src_stride_r,
+                                    fmoe_stream_t stream) {
+    FMOE_REQUIRE(elem_size == 1 || elem_size == 2, "fmoe_transpose_last2: element size must be 1 or 2");
+    FMOE_REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "fmoe_transpose_last2: negative extent");
+    if (batch == 0 || rows == 0 || cols == 0) return FMOE_OK;
+    FMOE_REQUIRE(src && dst, "fmoe_transpose_last2: NULL pointer");
+    FMOE_REQUIRE(src_stride_r >= cols, "fmoe_transpose_last2: source row stride %lld < cols %lld",
+                 (long long)src_stride_r, (long long)cols);
+    FMOE_REQUIRE(batch <= 65535 && (rows + 63) / 64 <= 65535, "fmoe_transpose_last2: grid too large");
+    dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64), (unsigned)batch);
+    if (elem_size == 2)
+        transpose_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, (uint16_t*)dst, rows, cols, src_stride_b, src_stride_r);
+    else
+        transpose_kernel<uint8_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint8_t*)src, (uint8_t*)dst, rows, cols, src_stride_b, src_stride_r);
+    return check_launch("fmoe_transpose_last2");
+}
+
 
 extern "C" int fmoe_version(void) { return 100; }
 

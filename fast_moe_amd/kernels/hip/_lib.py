@@ -19,7 +19,7 @@ EPI_NONE, EPI_SILU, EPI_SWIGLU = 0, 1, 2
 EXPORTED_SYMBOLS = (
     "fmoe_version", "fmoe_last_error", "fmoe_route_workspace_bytes", "fmoe_route_topk",
     "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_combine",
-    "fmoe_silu_mul",
+    "fmoe_silu_mul", "fmoe_transpose_last2",
 )
 
 
@@ -75,6 +75,9 @@ def load() -> ctypes.CDLL:
                                  c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p]
     lib.fmoe_silu_mul.restype = c_int
     lib.fmoe_silu_mul.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_void_p]
+    lib.fmoe_transpose_last2.restype = c_int
+    lib.fmoe_transpose_last2.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                         c_void_p]
     _lib = lib
     return lib
 

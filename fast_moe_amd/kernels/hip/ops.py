@@ -159,6 +159,21 @@ def quant_rows_fp8(a: torch.Tensor, apply_silu: bool = False, reciprocal_scale: 
     return q, scale.view(shape[:-1])
 
 
+def to_k_contiguous(w: torch.Tensor) -> torch.Tensor:
+    """[E, K, N] weight with N contiguous -> the same logical tensor as a view of [E, N, K]
+    storage (one transposing copy by fmoe_transpose_last2).  Other layouts are returned as is."""
+    if w.ndim != 3 or w.stride(2) != 1 or w.stride(1) == 1 or w.element_size() not in (1, 2):
+        return w
+    E, K, N = w.shape
+    if w.stride(1) < N:
+        return w
+    dst = torch.empty((E, N, K), dtype=w.dtype, device=w.device)
+    rc = _lib.load().fmoe_transpose_last2(w.data_ptr(), dst.data_ptr(), w.element_size(), E, K, N,
+                                          w.stride(0), w.stride(1), _stream(w))
+    _lib.check(rc, "fmoe_transpose_last2")
+    return dst.permute(0, 2, 1)
+
+
 # -------------------------------------------------------------- grouped GEMM
 def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, total_rows: int,
                  row_index: Optional[torch.Tensor] = None, index_div: int = 1,
@@ -188,6 +203,12 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     if offsets.numel() != E + 1:
         raise ValueError(f"grouped_gemm: offsets must have E+1={E + 1} entries")
     a = _rows_contiguous(a)
+    # N-contiguous weights of a useful size: one transposing copy buys the streaming kernel
+    # (the element-load kernel that reads them in place is correct but an order of magnitude slower)
+    if b.stride(2) == 1 and b.stride(1) != 1 and K % 16 == 0 and N % 8 == 0 and total_rows * N >= (1 << 22):
+        b = to_k_contiguous(b)
+        if b2 is not None:
+            b2 = to_k_contiguous(b2)
     offsets = _i64("offsets", offsets)
     if row_index is not None:
         row_index = _i64("row_index", row_index).view(-1)

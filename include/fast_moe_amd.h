@@ -89,7 +89,7 @@ int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K
  * ids (the generator of kernels/tests/moe_test.py:191-197,241: topk -> stable
  * sort -> scatter_add -> complete cumsum).  topk_idx values must lie in [0, E);
  * out-of-range ids are counted into no expert and reported through
- * `bad_count` (device int64, may be NULL).  Limits: E <= 65536, K <= 64.
+ * `bad_count` (device int64, may be NULL).  Limits: E <= 1024, K <= 64.
  */
 int fmoe_route_from_topk(const int64_t* topk_idx, int64_t T, int E, int K,
                          int64_t* lengths, int64_t* offsets, int64_t* gate_index,
@@ -214,6 +214,18 @@ int fmoe_combine(const void* value, int value_dtype, int64_t T, int K, int64_t D
  * tail of index_select_jagged_gating_bmm when its two inputs differ. */
 int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
                   fmoe_stream_t stream);
+
+/*
+ * dst[b, c, r] = src[b, r, c] for 1- or 2-byte elements: turns N-contiguous expert weights
+ * [E, K, N] into the K-contiguous [E, N, K] storage the fast GEMM path streams.  The reference
+ * has no counterpart (its Triton kernels read either layout through strides,
+ * kernels/triton/triton_moe.py:238-242); callers that keep weights N-contiguous transpose once
+ * per weight update, or per call as the Python wrapper does.
+ *   src  logical [batch, rows, cols], cols contiguous, element strides src_stride_b / src_stride_r
+ *   dst  [batch, cols, rows] contiguous
+ */
+int fmoe_transpose_last2(const void* src, void* dst, int elem_size, int64_t batch, int64_t rows,
+                         int64_t cols, int64_t src_stride_b, int64_t src_stride_r, fmoe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -383,3 +383,28 @@ def test_full_size_c3_c4_sampled_rows(fp8):
     common = set(int(e) for e in topk[4]) & set(int(e) for e in topk[5])
     for e in common:
         assert torch.equal(out[pos[(4, e)]], out[pos[(5, e)]])
+
+
+def test_n_contiguous_weights_take_the_transposing_fast_path():
+    """[E, K, N]-contiguous weights (the layout of kernels/tests/moe_test.py:205-209) of a useful
+    size are transposed once on the device and then streamed; the result equals the in-place
+    element-load kernel's and the oracle's."""
+    from fast_moe_amd.kernels import moe
+    from fast_moe_amd.kernels.hip import ops
+    L, E, K, Din, Dout = 8192, 8, 2, 512, 384
+    r = make_routing(L, E, K, seed=21)
+    x = randn((L, Din), 1)
+    w = weights(E, Din, Dout, 2, True, scale=Din ** -0.5)
+    assert w.is_contiguous()
+    wt = ops.to_k_contiguous(dev(w))
+    assert wt.stride(1) == 1 and torch.equal(wt.cpu(), w)
+    odd = weights(3, 70, 130, 4, True)           # extents that are not multiples of the 64 x 64 tile
+    assert torch.equal(ops.to_k_contiguous(dev(odd)).cpu(), odd)
+    q = (torch.arange(5 * 33 * 65) % 251).to(torch.uint8).view(5, 33, 65).view(torch.float8_e4m3fn)
+    assert torch.equal(ops.to_k_contiguous(dev(q)).cpu().view(torch.uint8), q.view(torch.uint8))
+    ref = o_moe.index_select_jagged_bmm(r["offsets"], r["index"], x.float(), w.float(), None)
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), None)
+        out_k = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), wt, None)
+    assert torch.equal(out, out_k)
+    assert_bf16_close(out, ref, rtol=1e-2, atol=1e-2, what="N-contiguous weights")
