@@ -60,6 +60,13 @@ __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __re
     }
 }
 
+__global__ __launch_bounds__(256) void silu_mul_f32_kernel(const float* __restrict__ a,
+                                                           const float* __restrict__ b,
+                                                           float* __restrict__ out, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = silu_f32(a[i]) * b[i];
+}
+
 // 64 x 64 tile transpose through LDS; reads and writes are both row-contiguous
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ src, T* __restrict__ dst,
@@ -113,10 +120,15 @@ extern "C" const char* fmoe_last_error(void) { return g_error; }
 
 extern "C" int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
                              fmoe_stream_t stream) {
-    FMOE_REQUIRE(dtype == FMOE_BF16, "fmoe_silu_mul: only bf16 is supported");
+    FMOE_REQUIRE(dtype == FMOE_BF16 || dtype == FMOE_F32, "fmoe_silu_mul: dtype must be bf16 or fp32");
     FMOE_REQUIRE(n >= 0, "fmoe_silu_mul: n < 0");
     if (n == 0) return FMOE_OK;
     FMOE_REQUIRE(a && b && out, "fmoe_silu_mul: NULL pointer");
+    if (dtype == FMOE_F32) {
+        silu_mul_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+            (const float*)a, (const float*)b, (float*)out, n);
+        return check_launch("fmoe_silu_mul");
+    }
     const int64_t threads = (n + 7) / 8;
     silu_mul_bf16_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, (hipStream_t)stream>>>(
         (const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, n);

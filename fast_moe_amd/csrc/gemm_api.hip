@@ -23,9 +23,10 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     FMOE_REQUIRE(d->num_experts >= 1 && d->n >= 1 && d->k >= 1,
                  "fmoe_grouped_gemm: need E, n, k >= 1 (E=%d n=%d k=%d)", d->num_experts, d->n, d->k);
     FMOE_REQUIRE(d->total_rows >= 0, "fmoe_grouped_gemm: total_rows < 0");
-    FMOE_REQUIRE(d->a_dtype == FMOE_BF16 || d->a_dtype == FMOE_E4M3,
-                 "fmoe_grouped_gemm: operands must be bf16 or e4m3 (got dtype %d)", d->a_dtype);
-    FMOE_REQUIRE(d->out_dtype == FMOE_BF16, "fmoe_grouped_gemm: output must be bf16");
+    FMOE_REQUIRE(d->a_dtype == FMOE_BF16 || d->a_dtype == FMOE_E4M3 || d->a_dtype == FMOE_F32,
+                 "fmoe_grouped_gemm: operands must be bf16, e4m3 or fp32 (got dtype %d)", d->a_dtype);
+    FMOE_REQUIRE(d->out_dtype == (d->a_dtype == FMOE_F32 ? FMOE_F32 : FMOE_BF16),
+                 "fmoe_grouped_gemm: output must be bf16 (fp32 for fp32 operands)");
     FMOE_REQUIRE(d->epilogue >= FMOE_EPI_NONE && d->epilogue <= FMOE_EPI_SWIGLU,
                  "fmoe_grouped_gemm: unknown epilogue %d", d->epilogue);
     if (d->total_rows == 0) return FMOE_OK;
@@ -37,6 +38,7 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     FMOE_REQUIRE(d->out_stride_row >= d->n, "fmoe_grouped_gemm: out row stride %lld < n %d",
                  (long long)d->out_stride_row, d->n);
     const bool fp8 = d->a_dtype == FMOE_E4M3;
+    const bool f32 = d->a_dtype == FMOE_F32;
     const bool swiglu = d->epilogue == FMOE_EPI_SWIGLU;
     if (swiglu) FMOE_REQUIRE(d->b2 != nullptr, "fmoe_grouped_gemm: SWIGLU needs b2");
     if (fp8) {
@@ -74,9 +76,11 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     p.out = (uint16_t*)d->out;
     p.out_stride = d->out_stride_row;
     p.n_tiles = 0;
-    p.vec_store = (d->n % 8 == 0) && (d->out_stride_row % 8 == 0) && aligned16(d->out);
+    // 16-byte stores: 8 bf16 (4 fp32) output columns at a time
+    const int vec_cols = f32 ? 4 : 8;
+    p.vec_store = (d->n % vec_cols == 0) && (d->out_stride_row % vec_cols == 0) && aligned16(d->out);
 
-    const int esize = fp8 ? 1 : 2;
+    const int esize = fp8 ? 1 : (f32 ? 4 : 2);
     const int chunk = 16 / esize;
     const bool fast = d->b_stride_k == 1 && (d->k % chunk) == 0 && aligned16(d->a) && aligned16(d->b) &&
                       (!swiglu || aligned16(d->b2)) && (d->a_stride_row % chunk) == 0 &&
@@ -87,9 +91,10 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     const bool big = d->total_rows / d->num_experts >= 96;
     // the ring kernel moves whole 64-byte K-slices by LDS-DMA and stores 16-byte groups
     const int slice = 64 / esize;
-    const bool ring = fast && big && !d->a_silu && (d->k % slice) == 0 && d->k / slice >= 3 &&
+    const bool ring = fast && big && !f32 && !d->a_silu && (d->k % slice) == 0 && d->k / slice >= 3 &&
                       p.vec_store && d->num_experts <= 1024 && d->total_rows < ((int64_t)1 << 31) * 128;
     const int sel = !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
     if (fp8) return run_gemm_fp8(p, d->epilogue, sel, stream);
+    if (f32) return run_gemm_f32(p, d->epilogue, d->a_silu != 0, sel, stream);
     return run_gemm_bf16(p, d->epilogue, d->a_silu != 0, sel, stream);
 }

@@ -7,9 +7,9 @@ namespace fmoe {
 
 int run_gemm_fp8(GemmParams& p, int epilogue, int sel, hipStream_t stream) {
     switch (epilogue) {
-        case FMOE_EPI_NONE: return dispatch_tile<true, FMOE_EPI_NONE, false>(p, sel, stream);
-        case FMOE_EPI_SILU: return dispatch_tile<true, FMOE_EPI_SILU, false>(p, sel, stream);
-        case FMOE_EPI_SWIGLU: return dispatch_tile<true, FMOE_EPI_SWIGLU, false>(p, sel, stream);
+        case FMOE_EPI_NONE: return dispatch_tile<kDtE4m3, FMOE_EPI_NONE, false>(p, sel, stream);
+        case FMOE_EPI_SILU: return dispatch_tile<kDtE4m3, FMOE_EPI_SILU, false>(p, sel, stream);
+        case FMOE_EPI_SWIGLU: return dispatch_tile<kDtE4m3, FMOE_EPI_SWIGLU, false>(p, sel, stream);
     }
     return fail(FMOE_ERR_ARGUMENT, "fmoe_grouped_gemm: unknown epilogue %d", epilogue);
 }

@@ -61,6 +61,7 @@ struct GemmParams {
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
 };
 
+constexpr int kDtBf16 = 0, kDtE4m3 = 1, kDtF32 = 2;
 constexpr int kGroupM = 4;   // row tiles per scheduling group
 constexpr int kNumXcd = 8;
 
@@ -94,6 +95,12 @@ __device__ __forceinline__ u32x4 silu_bf16x8(u32x4 v) {
         const float hi = silu_f32(__uint_as_float(v[j] & 0xffff0000u));
         v[j] = pack_bf16(lo, hi);
     }
+    return v;
+}
+
+__device__ __forceinline__ u32x4 silu_f32x4(u32x4 v) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = __float_as_uint(silu_f32(__uint_as_float(v[j])));
     return v;
 }
 
@@ -189,6 +196,55 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     }
 }
 
+// fp32 operands: fp32 bias and output, no intermediate rounding, exact SiLU.
+template <int FM, int FN, int TM, int TN, int EPI>
+__device__ __forceinline__ void gemm_epilogue_f32(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
+                                                  int n0, int64_t row0, int rows_valid, int wm, int wn,
+                                                  int lane) {
+    constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
+    constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
+    const int khalf = lane >> 5;
+    const float* bias = reinterpret_cast<const float*>(p.bias);
+    const float* bias2 = reinterpret_cast<const float*>(p.bias2);
+    float* out = reinterpret_cast<float*>(p.out);
+    const int64_t bias_row = (int64_t)expert * p.bias_se;
+#pragma unroll
+    for (int fn = 0; fn < FN_OUT; ++fn) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int nb = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + fn * 32 + 8 * g + 4 * khalf;
+            float bv[4], bv2[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int nc = nb + j < p.N ? nb + j : p.N - 1;
+                bv[j] = bias ? bias[bias_row + nc] : 0.0f;
+                bv2[j] = (SWIGLU && bias2) ? bias2[bias_row + nc] : 0.0f;
+            }
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) {
+                const int tile_row = wm * TM + fm * 32 + (lane & 31);
+                if (tile_row >= rows_valid) continue;
+                float* orow = out + (row0 + tile_row) * p.out_stride;
+                float o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float y = acc[fn][fm][4 * g + j] + bv[j];
+                    if (EPI == FMOE_EPI_SILU) y = silu_f32(y);
+                    if (SWIGLU) y = silu_f32(y) * (acc[fn + FN / 2][fm][4 * g + j] + bv2[j]);
+                    o[j] = y;
+                }
+                if (p.vec_store && nb + 3 < p.N) {
+                    *reinterpret_cast<f32x4*>(orow + nb) = f32x4{o[0], o[1], o[2], o[3]};
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (nb + j < p.N) orow[nb + j] = o[j];
+                }
+            }
+        }
+    }
+}
+
 // ----------------------------------------------------------- register-staged kernel
 template <int BM_, int BN_, int WGM_, int WGN_>
 struct TileCfg {
@@ -206,11 +262,14 @@ __device__ __forceinline__ int lds_off(int row, int chunk) {     // 128-byte row
     return row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4);
 }
 
-template <typename TL, bool FP8, int EPI, bool FAST, bool A_SILU>
+// DT: operand type, kDtBf16 / kDtE4m3 (bf16 output) or kDtF32 (fp32 operands, bias and output,
+// v_mfma_f32_32x32x2_f32: full fp32 products, no tf32).
+template <typename TL, int DT, int EPI, bool FAST, bool A_SILU>
 __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p) {
     constexpr int BM = TL::BM, BN = TL::BN, NT = TL::NT;
     constexpr int FM = TL::FM, FN = TL::FN, TM = TL::TM, TN = TL::TN;
-    constexpr int ESIZE = FP8 ? 1 : 2;
+    constexpr bool FP8 = DT == kDtE4m3, F32 = DT == kDtF32;
+    constexpr int ESIZE = FP8 ? 1 : (F32 ? 4 : 2);
     constexpr int CHUNK_ELEMS = 16 / ESIZE;         // elements per 16-byte chunk
     constexpr int BK = 128 / ESIZE;                 // elements per K-slice
     constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
@@ -351,12 +410,13 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
                     uint32_t v = 0;
                     if (k + j < p.K)
                         v = FP8 ? (uint32_t)xptr[i][k + j]
-                                : (uint32_t) reinterpret_cast<const uint16_t*>(xptr[i])[k + j];
+                            : F32 ? reinterpret_cast<const uint32_t*>(xptr[i])[k + j]
+                                  : (uint32_t) reinterpret_cast<const uint16_t*>(xptr[i])[k + j];
                     w[(j * ESIZE) >> 2] |= v << (8 * ((j * ESIZE) & 3));
                 }
                 xr[i] = u32x4{w[0], w[1], w[2], w[3]};
             }
-            if (A_SILU) xr[i] = silu_bf16x8(xr[i]);
+            if (A_SILU) xr[i] = F32 ? silu_f32x4(xr[i]) : silu_bf16x8(xr[i]);
         }
 #pragma unroll
         for (int i = 0; i < WP; ++i) {
@@ -373,7 +433,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
                     if (k + j < p.K) {
                         const int64_t off = (int64_t)(k + j) * p.b_sk;
                         v = FP8 ? (uint32_t)wptr[i][off]
-                                : (uint32_t) reinterpret_cast<const uint16_t*>(wptr[i])[off];
+                            : F32 ? reinterpret_cast<const uint32_t*>(wptr[i])[off]
+                                  : (uint32_t) reinterpret_cast<const uint16_t*>(wptr[i])[off];
                     }
                     w[(j * ESIZE) >> 2] |= v << (8 * ((j * ESIZE) & 3));
                 }
@@ -420,7 +481,29 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
         if (kt + 1 < KT) load_global(kt + 1);
         const uint8_t* sx = smem + cur * TL::STAGE_BYTES;
         const uint8_t* sw = sx + BM * 128;
-        if (!FP8) {
+        if (F32) {
+            // a 16-byte chunk holds 4 consecutive k of one row; MFMA j of a chunk pair contracts
+            // element j of the low-half lanes' chunk with element j of the high-half lanes' chunk
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int chunk = 2 * s + khalf;
+                u32x4 wf[FN], xf[FM];
+#pragma unroll
+                for (int fn = 0; fn < FN; ++fn)
+                    wf[fn] = *reinterpret_cast<const u32x4*>(sw + lds_off(wfrag_row[fn], chunk));
+#pragma unroll
+                for (int fm = 0; fm < FM; ++fm)
+                    xf[fm] = *reinterpret_cast<const u32x4*>(sx + lds_off(xfrag_row[fm], chunk));
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int fn = 0; fn < FN; ++fn)
+#pragma unroll
+                        for (int fm = 0; fm < FM; ++fm)
+                            acc[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                __uint_as_float(wf[fn][j]), __uint_as_float(xf[fm][j]), acc[fn][fm], 0, 0, 0);
+            }
+        } else if (!FP8) {
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const int chunk = 2 * s + khalf;
@@ -468,7 +551,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
         __syncthreads();
     }
 
-    gemm_epilogue<FM, FN, TM, TN, FP8, EPI>(p, acc, expert, n0, row0, rows_valid, wm, wn, lane);
+    if constexpr (F32)
+        gemm_epilogue_f32<FM, FN, TM, TN, EPI>(p, acc, expert, n0, row0, rows_valid, wm, wn, lane);
+    else
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI>(p, acc, expert, n0, row0, rows_valid, wm, wn, lane);
 }
 
 // --------------------------------------------------------------------- ring kernel
@@ -795,11 +881,11 @@ int reserve_lds(Kern kern, int bytes, bool& done) {
     return FMOE_OK;
 }
 
-template <typename TL, bool FP8, int EPI, bool FAST, bool A_SILU>
+template <typename TL, int DT, int EPI, bool FAST, bool A_SILU>
 int launch_gemm(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
-    auto kern = grouped_gemm_kernel<TL, FP8, EPI, FAST, A_SILU>;
+    auto kern = grouped_gemm_kernel<TL, DT, EPI, FAST, A_SILU>;
     static bool attr_done = false;
     if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
     const int64_t max_m_tiles = p.total_rows / TL::BM + p.E;
@@ -828,20 +914,21 @@ int launch_ring(GemmParams p, hipStream_t stream) {
     return check_launch("fmoe_grouped_gemm");
 }
 
-template <bool FP8, int EPI, bool A_SILU>
+template <int DT, int EPI, bool A_SILU>
 int dispatch_tile(const GemmParams& p, int sel, hipStream_t stream) {
     switch (sel) {
         case kSelRing:
-            if constexpr (!A_SILU) return launch_ring<FP8, EPI>(p, stream);
-            else return launch_gemm<TileBig, FP8, EPI, true, A_SILU>(p, stream);
-        case kSelStagedBig: return launch_gemm<TileBig, FP8, EPI, true, A_SILU>(p, stream);
-        case kSelStagedSmall: return launch_gemm<TileSmall, FP8, EPI, true, A_SILU>(p, stream);
-        default: return launch_gemm<TileSmall, FP8, EPI, false, A_SILU>(p, stream);
+            if constexpr (!A_SILU && DT != kDtF32) return launch_ring<DT == kDtE4m3, EPI>(p, stream);
+            else return launch_gemm<TileBig, DT, EPI, true, A_SILU>(p, stream);
+        case kSelStagedBig: return launch_gemm<TileBig, DT, EPI, true, A_SILU>(p, stream);
+        case kSelStagedSmall: return launch_gemm<TileSmall, DT, EPI, true, A_SILU>(p, stream);
+        default: return launch_gemm<TileSmall, DT, EPI, false, A_SILU>(p, stream);
     }
 }
 
-// Entry points of the two translation units.
+// Entry points of the translation units (one per operand type).
 int run_gemm_bf16(GemmParams& p, int epilogue, bool a_silu, int sel, hipStream_t stream);
 int run_gemm_fp8(GemmParams& p, int epilogue, int sel, hipStream_t stream);
+int run_gemm_f32(GemmParams& p, int epilogue, bool a_silu, int sel, hipStream_t stream);
 
 }  // namespace fmoe

@@ -182,13 +182,14 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  a_scale: Optional[torch.Tensor] = None, b_scale: Optional[torch.Tensor] = None,
                  b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
-    strides (bf16) or float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns bf16
-    [total_rows, N]."""
+    strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
+    [total_rows, N] in bf16 (fp32 for fp32 operands)."""
     dev = _need_cuda("grouped_gemm", offsets, a, b, row_index, bias, b2, bias2, a_scale, b_scale, b2_scale)
     fp8 = a.dtype == FP8_DTYPE
-    if not fp8 and a.dtype != torch.bfloat16:
+    if not fp8 and a.dtype not in (torch.bfloat16, torch.float32):
         raise NotImplementedError(
-            f"grouped_gemm: the HIP kernels take bf16 or float8_e4m3fn operands, got {a.dtype}")
+            f"grouped_gemm: the HIP kernels take bf16, fp32 or float8_e4m3fn operands, got {a.dtype}")
+    out_dtype = torch.float32 if a.dtype == torch.float32 else torch.bfloat16
     if b.dtype != a.dtype or (b2 is not None and b2.dtype != a.dtype):
         raise ValueError("grouped_gemm: A and B must share a dtype")
     if b.ndim != 3:
@@ -214,15 +215,15 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
         row_index = _i64("row_index", row_index).view(-1)
         if row_index.numel() != total_rows:
             raise ValueError("grouped_gemm: row_index must have total_rows entries")
-    out = torch.empty((total_rows, N), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((total_rows, N), dtype=out_dtype, device=dev)
     if total_rows == 0:
         return out
 
     def bias_ok(t):
         if t is None:
             return None
-        if t.dtype != torch.bfloat16 or tuple(t.shape) != (E, N):
-            raise ValueError("grouped_gemm: bias must be bf16 [E, N]")
+        if t.dtype != out_dtype or tuple(t.shape) != (E, N):
+            raise ValueError(f"grouped_gemm: bias must be {out_dtype} [E, N]")
         return _rows_contiguous(t)
 
     bias, bias2 = bias_ok(bias), bias_ok(bias2)
@@ -246,7 +247,7 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.offsets = offsets.data_ptr()
     d.row_index = _ptr(row_index)
     d.a = a.data_ptr()
-    d.a_dtype = FMOE_E4M3 if fp8 else FMOE_BF16
+    d.a_dtype = FMOE_E4M3 if fp8 else _DTYPE_CODE[a.dtype]
     d.a_silu = int(a_silu)
     d.a_stride_row = a.stride(0)
     d.a_stride_e = a_expert_stride
@@ -260,7 +261,7 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.bias2 = _ptr(bias2)
     d.bias_stride_e = bias.stride(0) if bias is not None else (bias2.stride(0) if bias2 is not None else 0)
     d.epilogue = epilogue
-    d.out_dtype = FMOE_BF16
+    d.out_dtype = _DTYPE_CODE[out_dtype]
     d.out = out.data_ptr()
     d.out_stride_row = out.stride(0)
     rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
@@ -308,12 +309,13 @@ def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[to
 
 
 def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """``silu(a) * b`` element-wise (bf16, contiguous, same shape)."""
+    """``silu(a) * b`` element-wise (bf16 or fp32, same shape)."""
     _need_cuda("silu_mul", a, b)
-    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16 or a.shape != b.shape:
-        raise ValueError("silu_mul: two bf16 tensors of one shape expected")
+    if a.dtype not in _DTYPE_CODE or b.dtype != a.dtype or a.shape != b.shape:
+        raise ValueError("silu_mul: two bf16 (or two fp32) tensors of one shape expected")
     a, b = a.contiguous(), b.contiguous()
     out = torch.empty_like(a)
-    rc = _lib.load().fmoe_silu_mul(a.data_ptr(), b.data_ptr(), out.data_ptr(), FMOE_BF16, a.numel(), _stream(a))
+    rc = _lib.load().fmoe_silu_mul(a.data_ptr(), b.data_ptr(), out.data_ptr(), _DTYPE_CODE[a.dtype], a.numel(),
+                                   _stream(a))
     _lib.check(rc, "fmoe_silu_mul")
     return out

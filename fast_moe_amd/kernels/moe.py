@@ -9,7 +9,7 @@ of /root/reference/kernels/moe.py:39-292.  Differences, all on purpose:
 * forward only: inputs that require grad raise unless grad mode is off.
 * ``max_seq_len`` is accepted and ignored: tile scheduling reads ``offsets`` on
   the device, so no host synchronisation is needed to obtain it.
-* operands must be bf16 CUDA tensors (fp32 for ``mul_merge_k_add``).
+* operands must be bf16 or fp32 CUDA tensors (fp32 runs true-fp32 MFMA, no tf32).
 """
 from __future__ import annotations
 

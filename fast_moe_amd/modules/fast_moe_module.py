@@ -77,8 +77,8 @@ class FastMoELayer(nn.Module):
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
             raise RuntimeError("FastMoELayer: the HIP back-end is forward-only; call it under "
                                "torch.no_grad() / torch.inference_mode()")
-        if x.dtype != torch.bfloat16:
-            raise NotImplementedError(f"FastMoELayer: the HIP kernels take bf16 activations, got {x.dtype}")
+        if x.dtype not in (torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"FastMoELayer: the HIP kernels take bf16 or fp32 activations, got {x.dtype}")
         original_shape = x.shape
         k = num_experts_per_tok
         r = self.route(x, k)

@@ -160,8 +160,8 @@ typedef struct fmoe_gemm_desc {
     const int64_t* row_index; /* [total_rows] or NULL                             */
 
     const void* a;          /* [a_rows, k] (or [a_rows, E, k] with a_stride_e)    */
-    int32_t a_dtype;        /* FMOE_BF16 | FMOE_E4M3                              */
-    int32_t a_silu;         /* apply SiLU to A elements on load (bf16 only)       */
+    int32_t a_dtype;        /* FMOE_BF16 | FMOE_E4M3 | FMOE_F32                   */
+    int32_t a_silu;         /* apply SiLU to A elements on load (bf16 / fp32)      */
     int64_t a_stride_row;
     int64_t a_stride_e;     /* 0, or per-expert offset for the 3D variant         */
     const float* a_scale;   /* [a_rows] multiplier scales (FMOE_E4M3)             */
@@ -177,7 +177,7 @@ typedef struct fmoe_gemm_desc {
     int64_t bias_stride_e;
 
     int32_t epilogue;       /* enum fmoe_epilogue                                 */
-    int32_t out_dtype;      /* FMOE_BF16                                          */
+    int32_t out_dtype;      /* FMOE_BF16; FMOE_F32 iff a_dtype is FMOE_F32        */
     void* out;              /* [total_rows, n]                                    */
     int64_t out_stride_row;
 } fmoe_gemm_desc;
@@ -209,7 +209,7 @@ int fmoe_combine(const void* value, int value_dtype, int64_t T, int K, int64_t D
                  int64_t gates_stride_col, const int64_t* gates_index, void* out, int out_dtype,
                  fmoe_stream_t stream);
 
-/* out[i] = silu(a[i]) * b[i] over n bf16 elements with the reference's rounding
+/* out[i] = silu(a[i]) * b[i] over n bf16 (or fp32) elements with the reference's rounding
  * points (F.silu(alpha) * beta, kernels/pytorch/moe.py:221): the element-wise
  * tail of index_select_jagged_gating_bmm when its two inputs differ. */
 int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,

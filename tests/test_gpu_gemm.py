@@ -267,7 +267,7 @@ def test_forward_only_and_dtype_errors():
         moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, None)
     with pytest.raises(NotImplementedError):
         with torch.no_grad():
-            moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x.float(), w.float(), None)
+            moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x.half(), w.half(), None)
 
 
 # ------------------------------------------------------------- ring-kernel specifics
@@ -408,3 +408,54 @@ def test_n_contiguous_weights_take_the_transposing_fast_path():
         out_k = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), wt, None)
     assert torch.equal(out, out_k)
     assert_bf16_close(out, ref, rtol=1e-2, atol=1e-2, what="N-contiguous weights")
+
+
+# ------------------------------------------------------------------------ fp32
+@pytest.mark.parametrize("L,E,K,Din,Dout", GRID[1::4])
+@pytest.mark.parametrize("contiguous", [True, False])
+@pytest.mark.parametrize("has_bias", [True, False])
+def test_index_select_jagged_bmm_fp32_reference_grid(L, E, K, Din, Dout, contiguous, has_bias):
+    """fp32 half of kernels/tests/moe_test.py:35-84 (allow_tf32 off): default fp32 assert_close."""
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=L + E + 1)
+    x = uniform((L, Din), 1, torch.float32)
+    w = uniform((E, Din, Dout), 2, torch.float32)
+    if not contiguous:
+        w = w.transpose(1, 2).contiguous().transpose(1, 2)
+    b = uniform((E, Dout), 3, torch.float32) if has_bias else None
+    ref = o_moe.index_select_jagged_bmm(r["offsets"], r["index"], x, w, b)
+    with torch.no_grad():
+        out = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), dev(x), dev(w), dev(b))
+    assert out.dtype == torch.float32
+    torch.testing.assert_close(out.cpu(), ref)
+
+
+def test_fp32_swiglu_gating_3d_and_combine():
+    from fast_moe_amd.kernels import moe
+    L, E, K, Din, Dout = 700, 8, 2, 64, 96
+    f32 = torch.float32
+    r = make_routing(L, E, K, seed=31)
+    x, x2 = uniform((L, Din), 1, f32), uniform((L, Din), 4, f32)
+    w, wp = uniform((E, Din, Dout), 2, f32), uniform((E, Din, Dout), 5, f32)
+    b, bp = uniform((E, Dout), 3, f32), uniform((E, Dout), 6, f32)
+    a = [dev(r["offsets"]), dev(r["index"])]
+    with torch.no_grad():
+        sw = moe.index_select_jagged_bmm_swiglu(0, *a, dev(x), dev(w), dev(b), dev(wp), dev(bp))
+        gt = moe.index_select_jagged_gating_bmm(0, *a, dev(x), dev(x2), dev(w), dev(b), dev(wp), dev(bp))
+    torch.testing.assert_close(sw.cpu(), o_moe.index_select_jagged_bmm_swiglu(r["offsets"], r["index"], x, w, b, wp, bp),
+                               rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(gt.cpu(), o_moe.index_select_jagged_gating_bmm(r["offsets"], r["index"], x, x2, w, wp, b, bp),
+                               rtol=1e-5, atol=1e-5)
+    x3 = uniform((L, E, Din), 7, f32)
+    with torch.no_grad():
+        o3 = moe.index_select_jagged_bmm_3D(0, *a, dev(x3), dev(w), dev(b))
+    torch.testing.assert_close(o3.cpu(), o_moe.index_select_jagged_bmm_3D(r["offsets"], r["index"], x3, w, b))
+    # SiLU-on-load GEMM + merge
+    g = torch.Generator().manual_seed(3)
+    gates = torch.rand(L, K, generator=g)
+    jag = uniform((L * K, Din), 8, f32)
+    ref = o_moe.silu_jagged_bmm_combine(r["offsets"], jag, w, b, r["token_index"], K, gates, r["gate_index"], True)
+    with torch.no_grad():
+        out = moe.silu_jagged_bmm_combine(0, dev(r["offsets"]), dev(jag), dev(w), dev(b), dev(r["token_index"]),
+                                          dev(r["reverse_index"]), dev(gates), dev(r["gate_index"]), has_silu=True)
+    torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-5)

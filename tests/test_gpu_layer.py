@@ -126,3 +126,38 @@ def test_swiglu_moe_bf16_and_fp8_composition(T, E, K, D, H):
     # fp8 against the oracle's own fp8 path: 3e-2 relative (of the output scale for small entries)
     scale8 = ref8.float().abs().max().item()
     assert_bf16_close(y8, ref8, rtol=3e-2, atol=3e-2 * scale8, what="swiglu fp8")
+
+
+@pytest.mark.parametrize("B,S,D,H,O,E,k", [(4, 4, 16, 16, 16, 4, 1), (8, 16, 32, 32, 16, 8, 2), (4, 512, 1024, 4096, 1024, 8, 2)])
+def test_layer_fp32_matches_oracle(B, S, D, H, O, E, k):
+    """modules/tests/test_kernel_parity.py:29-90 (fp32, atol 1e-4) and configuration C1 of the
+    baseline (fp32, 8 experts, top-2, [4, 512, 1024] tokens, hidden 4096) against the oracle's
+    PyTorch-kernel path on the CPU."""
+    from fast_moe_amd import FastMoELayer
+    torch.manual_seed(0)
+    layer = FastMoELayer(D, H, O, E, dtype=torch.float32)
+    g = torch.Generator().manual_seed(0)
+    with torch.no_grad():
+        layer._experts_hidden_w.copy_(torch.randn(E, H, D, generator=g) * D ** -0.5)
+        layer._experts_w.copy_(torch.randn(E, O, H, generator=g) * H ** -0.5)
+        layer.gate.gate.weight.copy_(torch.randn(E, D, generator=g) * D ** -0.5)
+        layer.gate.gate.bias.zero_()
+    x = torch.randn(B, S, D, generator=g)
+    sd = {n: v.detach().clone() for n, v in layer.state_dict().items()}
+    gpu = layer.cuda()
+    with torch.no_grad():
+        y = gpu(x.cuda(), k)
+        scores = gpu.gate(x.cuda()).reshape(-1, E).cpu()
+    ref, r = o_layer.moe_layer_forward(x, sd["gate.gate.weight"], sd["gate.gate.bias"], sd["_experts_hidden_w"],
+                                       sd["_experts_hidden_bias"], sd["_experts_w"], sd["_experts_bias"], k)
+    # routing from the GPU's own gate probabilities (a last-bit softmax difference may flip a near-tie)
+    r2 = o_layer.route_scores(scores, k)
+    if not torch.equal(r2["topk_idx"], r["topk_idx"]):
+        xf = x.reshape(-1, D)
+        hidden = o_moe.index_select_jagged_bmm(r2["offsets"], r2["gate_index"].view(-1, k), xf,
+                                               sd["_experts_hidden_w"].permute(0, 2, 1), sd["_experts_hidden_bias"])
+        ref = o_moe.silu_jagged_bmm_combine(r2["offsets"], hidden, sd["_experts_w"].permute(0, 2, 1),
+                                            sd["_experts_bias"], r2["token_index"], k, r2["gates"],
+                                            r2["gate_index"]).view(B, S, O)
+    assert y.dtype == torch.float32
+    torch.testing.assert_close(y.cpu(), ref, atol=1e-4, rtol=1e-4)
