@@ -82,9 +82,12 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     d.num_experts, d.n, d.k = 4, 0, 8
     assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
     assert b"n, k >= 1" in lib.fmoe_last_error()
-    d.n, d.total_rows, d.a_dtype, d.out_dtype = 8, 16, 0, 1
+    d.n, d.total_rows, d.a_dtype, d.out_dtype = 8, 16, 7, 1
     assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
-    assert b"bf16 or e4m3" in lib.fmoe_last_error()
+    assert b"bf16, e4m3 or fp32" in lib.fmoe_last_error()
+    d.a_dtype = 0                                    # fp32 operands need an fp32 output
+    assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
+    assert b"fp32 for fp32 operands" in lib.fmoe_last_error()
     # routing: K > E, K > 64, workspace too small
     args = [None] * 7
     assert lib.fmoe_route_topk(None, 0, 4, 8, 80, 1, *args, None, 0, None) == 1
