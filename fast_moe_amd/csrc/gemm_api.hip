@@ -15,6 +15,18 @@ int compute_units() {
     }
     return cached[dev];
 }
+
+int lds_per_block() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || n <= 0) n = 65536;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
 }  // namespace fmoe
 
 extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_) {
@@ -91,8 +103,12 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     const bool big = d->total_rows / d->num_experts >= 96;
     // the ring kernel moves whole 64-byte K-slices by LDS-DMA and stores 16-byte groups
     const int slice = 64 / esize;
+    // ... and addresses rows as a 64-bit base per expert plus a 32-bit byte offset
+    const int64_t span32 = ((int64_t)1 << 32) - 4096;
+    const bool near = d->a_rows * d->a_stride_row * esize + (int64_t)d->k * esize < span32 &&
+                      (int64_t)d->n * d->b_stride_n * esize + (int64_t)d->k * esize < span32;
     const bool ring = fast && big && !f32 && !d->a_silu && (d->k % slice) == 0 && d->k / slice >= 3 &&
-                      p.vec_store && d->num_experts <= 1024 && d->total_rows < ((int64_t)1 << 31) * 128;
+                      p.vec_store && d->num_experts <= 1024 && d->total_rows < ((int64_t)1 << 31) * 128 && near;
     const int sel = !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
     if (fp8) return run_gemm_fp8(p, d->epilogue, sel, stream);
     if (f32) return run_gemm_f32(p, d->epilogue, d->a_silu != 0, sel, stream);

@@ -558,22 +558,28 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
 }
 
 // --------------------------------------------------------------------- ring kernel
-template <int BM_, int BN_, int WGM_, int WGN_, int STAGES_>
+// NREG_ == 0: 4 slots, one K-slice issued per step, schedule tables in LDS (E <= 1024).
+// NREG_  > 0: 5 slots (all 160 KB of LDS), K-slices issued in pairs so that the two
+//             instructions touching the halves of a 128-byte line are adjacent and reach L2
+//             as one full-line request; the schedule tables live in 3 * NREG_ registers of
+//             every wave (E <= 64 * NREG_, total_rows < 2^31, K-slices per tile even).
+template <int BM_, int BN_, int WGM_, int WGN_, int NREG_>
 struct RingCfg {
-    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_, STAGES = STAGES_;
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_, NREG = NREG_;
+    static constexpr bool PAIR = NREG_ > 0;
+    static constexpr int STAGES = PAIR ? 5 : 4;
     static constexpr int NW = WGM * WGN;
     static constexpr int NT = kWave * NW;
     static constexpr int TM = BM / WGM, TN = BN / WGN;
     static constexpr int FM = TM / 32, FN = TN / 32;
     static constexpr int STAGE_BYTES = (BM + BN) * 64;          // 64-byte K-slice per row
     static constexpr int RING_BYTES = STAGES * STAGE_BYTES;
-    static constexpr int kMaxExperts = 1024;
+    static constexpr int kMaxExperts = PAIR ? 64 * NREG_ : 1024;
     static constexpr int TAB_OFF = RING_BYTES;                   // int32 [E+1] row-tile prefix
     static constexpr int OFF_OFF = RING_BYTES + 4128;            // int64 [E+1] clamped offsets
-    static constexpr int LDS_BYTES = OFF_OFF + (kMaxExperts + 1) * 8 + 8;
+    static constexpr int LDS_BYTES = PAIR ? RING_BYTES : OFF_OFF + (kMaxExperts + 1) * 8 + 8;
     static constexpr int XI = BM / 16 / NW, WI = BN / 16 / NW;   // LDS-DMA instructions per lane per slice
     static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "DMA passes must be whole");
-    static_assert(STAGES == 3 || STAGES == 4, "the wait ladder below covers 3 or 4 slots");
     static_assert(TM % 32 == 0 && TN % 64 == 0, "wave tile must hold whole 32x32 fragments, FN even");
 };
 
@@ -581,12 +587,16 @@ __device__ __forceinline__ int lds_off64(int row, int chunk) {   // 64-byte rows
     return row * 64 + ((chunk ^ ((row >> 2) & 3)) << 4);
 }
 
-// One 16-byte-per-lane global -> LDS transfer.  The 64 lanes land on 1 KB of LDS starting at
-// the wave-uniform byte address lds_addr (M0), lane l at +16*l.  Issued as inline asm so
-// that the waits on it stay under this kernel's control (vmcnt is counted by hand below).
-__device__ __forceinline__ void dma16(const void* gptr, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n"
-                 :: "v"(gptr), "s"(lds_addr) : "memory");
+// One 16-byte-per-lane global -> LDS transfer from base + voff: a wave-uniform base in
+// SGPRs plus a 32-bit per-lane offset, so that stepping along K costs scalar adds only (VALU
+// instructions queue behind the MFMAs of the SIMD's other wave).  No immediate offset: the
+// hardware would add it to the LDS address as well.  The 64 lanes land on 1 KB of LDS
+// starting at the wave-uniform byte address lds_addr (M0), lane l at +16*l.  Issued as
+// inline asm so that the waits on it stay under this kernel's control (vmcnt is counted by
+// hand below).
+__device__ __forceinline__ void dma16(const uint8_t* base, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n"
+                 :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");
 }
 
 template <int N>
@@ -594,10 +604,16 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+__device__ __forceinline__ int uniform_lane(int v, int src_lane) {
+    return __builtin_amdgcn_readfirstlane(wave_bcast(v, src_lane));
+}
+
 template <typename TL, bool FP8, int EPI>
 __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmParams p) {
     constexpr int BM = TL::BM, BN = TL::BN, NW = TL::NW, STAGES = TL::STAGES;
     constexpr int FM = TL::FM, FN = TL::FN, TM = TL::TM, TN = TL::TN;
+    constexpr bool PAIR = TL::PAIR;
+    constexpr int NR = PAIR ? TL::NREG : 1;
     constexpr int ESIZE = FP8 ? 1 : 2;
     constexpr int BK = 64 / ESIZE;
     constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
@@ -617,26 +633,51 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 
     // ------------------------------------------------------------ schedule tables
     const int64_t R = p.total_rows;
-    if (wave == 0) {
+    int total_m;
+    // register tables: lane l of entry i describes expert 64 * i + l
+    int r_first[NR], r_lo[NR], r_len[NR];     // first row tile, first row, rows
+    if constexpr (PAIR) {
         int run = 0;
-        for (int e0 = 0; e0 <= p.E; e0 += kWave) {
-            const int e = e0 + lane;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const int e = i * kWave + lane;
             int64_t lo = 0, len = 0;
-            if (e <= p.E) lo = clamp_i64(p.offsets[e], 0, R);
             if (e < p.E) {
+                lo = clamp_i64(p.offsets[e], 0, R);
                 const int64_t hi = clamp_i64(p.offsets[e + 1], 0, R);
                 len = hi > lo ? hi - lo : 0;
             }
             const int tiles = (int)((len + BM - 1) / BM);
             const int inc = wave_inclusive_scan(tiles);
-            if (e < p.E) s_tab[e + 1] = run + inc;
-            if (e <= p.E) s_off[e] = lo;
-            run += wave_bcast(inc, kWave - 1);
+            r_first[i] = run + inc - tiles;
+            r_lo[i] = (int)lo;
+            r_len[i] = (int)len;
+            run += uniform_lane(inc, kWave - 1);
         }
-        if (lane == 0) s_tab[0] = 0;
+        total_m = run;
+    } else {
+        if (wave == 0) {
+            int run = 0;
+            for (int e0 = 0; e0 <= p.E; e0 += kWave) {
+                const int e = e0 + lane;
+                int64_t lo = 0, len = 0;
+                if (e <= p.E) lo = clamp_i64(p.offsets[e], 0, R);
+                if (e < p.E) {
+                    const int64_t hi = clamp_i64(p.offsets[e + 1], 0, R);
+                    len = hi > lo ? hi - lo : 0;
+                }
+                const int tiles = (int)((len + BM - 1) / BM);
+                const int inc = wave_inclusive_scan(tiles);
+                if (e < p.E) s_tab[e + 1] = run + inc;
+                if (e <= p.E) s_off[e] = lo;
+                run += wave_bcast(inc, kWave - 1);
+            }
+            if (lane == 0) s_tab[0] = 0;
+        }
+        __syncthreads();
+        total_m = s_tab[p.E];
+        r_first[0] = r_lo[0] = r_len[0] = 0;
     }
-    __syncthreads();
-    const int total_m = s_tab[p.E];
     const int64_t total_tiles = (int64_t)total_m * p.n_tiles;
     const int nslots = gridDim.x / kNumXcd;
     const int64_t per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
@@ -655,16 +696,39 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         const int mt = first_m + within % gsize;
         TileInfo t;
         t.nt = within / gsize;
-        int lo = 0, hi = p.E;
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (s_tab[mid] <= mt) lo = mid; else hi = mid;
+        if constexpr (PAIR) {
+            // the tile's expert = number of experts whose row tiles all precede mt
+            int cnt = 0;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int e = i * kWave + lane;
+                const bool before = e < p.E && r_first[i] + (r_len[i] + BM - 1) / BM <= mt;
+                cnt += __builtin_popcountll(__ballot(before));
+            }
+            cnt = __builtin_amdgcn_readfirstlane(cnt);
+            const int ri = cnt >> 6, rl = cnt & 63;
+            int vf = r_first[0], vl = r_lo[0], vn = r_len[0];
+#pragma unroll
+            for (int i = 1; i < NR; ++i)
+                if (ri == i) { vf = r_first[i]; vl = r_lo[i]; vn = r_len[i]; }
+            const int first = uniform_lane(vf, rl), lo = uniform_lane(vl, rl), len = uniform_lane(vn, rl);
+            const int skip = (mt - first) * BM;
+            t.expert = cnt;
+            t.row0 = (int64_t)lo + skip;
+            const int left = len - skip;
+            t.rows_valid = left < BM ? left : BM;
+        } else {
+            int lo = 0, hi = p.E;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (s_tab[mid] <= mt) lo = mid; else hi = mid;
+            }
+            t.expert = lo;
+            const int64_t e_lo = s_off[lo], e_hi = s_off[lo + 1];
+            t.row0 = e_lo + (int64_t)(mt - s_tab[lo]) * BM;
+            const int64_t left = (e_hi > e_lo ? e_hi : e_lo) - t.row0;
+            t.rows_valid = (int)(left < BM ? left : BM);
         }
-        t.expert = lo;
-        const int64_t e_lo = s_off[lo], e_hi = s_off[lo + 1];
-        t.row0 = e_lo + (int64_t)(mt - s_tab[lo]) * BM;
-        const int64_t left = (e_hi > e_lo ? e_hi : e_lo) - t.row0;
-        t.rows_valid = (int)(left < BM ? left : BM);
         return t;
     };
 
@@ -694,40 +758,47 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             ridx[i] = p.row_index ? p.row_index[r] : r;
         }
     };
-    const uint8_t* xptr[XI];
-    const uint8_t* wptr[WI];
+    // per-lane byte offsets of the rows this lane fetches, relative to wave-uniform bases
+    uint32_t xoff[XI], woff[WI];
+    const uint8_t* xbase = p.a;
+    const uint8_t* wbase[WI];
+    static_assert(!SWIGLU || (BN / 2) % (16 * NW) == 0, "a DMA instruction must not straddle gate and up rows");
     auto make_ptrs = [&](const TileInfo& t, const int64_t* ridx) {
-        const uint8_t* a_base = p.a + (int64_t)t.expert * p.a_stride_e * ESIZE;
+        const int expert = __builtin_amdgcn_readfirstlane(t.expert);
+        xbase = p.a + (int64_t)expert * p.a_stride_e * ESIZE;
         const int n0 = t.nt * BN_OUT;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             int64_t s = ridx[i];
             if (p.row_index) s = p.index_shift >= 0 ? (s >> p.index_shift) : s / p.index_div;
             s = clamp_i64(s, 0, p.a_rows - 1);
-            xptr[i] = a_base + s * (p.a_stride_row * ESIZE) + xsw[i];
+            xoff[i] = (uint32_t)(s * (p.a_stride_row * ESIZE)) + xsw[i];
         }
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
-            const uint8_t* base;
-            int n;
-            if (SWIGLU) {
-                base = wrow[i] < BN / 2 ? p.b : p.b2;
-                n = n0 + (wrow[i] < BN / 2 ? wrow[i] : wrow[i] - BN / 2);
-            } else {
-                base = p.b;
-                n = n0 + wrow[i];
-            }
+            const bool up = SWIGLU && i * NW * 16 >= BN / 2;
+            int n = n0 + wrow[i] - (up ? BN / 2 : 0);
             n = n < p.N ? n : p.N - 1;
-            wptr[i] = base + ((int64_t)t.expert * p.b_se + (int64_t)n * p.b_sn) * ESIZE + wsw[i];
+            wbase[i] = (up ? p.b2 : p.b) + (int64_t)expert * p.b_se * ESIZE;
+            woff[i] = (uint32_t)((int64_t)n * p.b_sn * ESIZE) + wsw[i];
         }
     };
-    auto issue = [&](int kt, int slot_i) {
-        const uint32_t sbase = lds_base + slot_i * TL::STAGE_BYTES;
+    // one K-slice into slot sa; in pair mode also the following slice into slot sb, the two
+    // 64-byte halves of every row's 128 bytes requested by adjacent instructions
+    auto issue = [&](int kt, int sa, int sb) {
+        const uint32_t abase = lds_base + sa * TL::STAGE_BYTES;
+        const uint32_t bbase = lds_base + sb * TL::STAGE_BYTES;
         const int64_t koff = (int64_t)kt * 64;
 #pragma unroll
-        for (int i = 0; i < XI; ++i) dma16(xptr[i] + koff, sbase + (i * NW + wave) * 1024);
+        for (int i = 0; i < XI; ++i) {
+            dma16(xbase + koff, xoff[i], abase + (i * NW + wave) * 1024);
+            if (PAIR) dma16(xbase + koff + 64, xoff[i], bbase + (i * NW + wave) * 1024);
+        }
 #pragma unroll
-        for (int i = 0; i < WI; ++i) dma16(wptr[i] + koff, sbase + BM * 64 + (i * NW + wave) * 1024);
+        for (int i = 0; i < WI; ++i) {
+            dma16(wbase[i] + koff, woff[i], abase + BM * 64 + (i * NW + wave) * 1024);
+            if (PAIR) dma16(wbase[i] + koff + 64, woff[i], bbase + BM * 64 + (i * NW + wave) * 1024);
+        }
     };
 
     int wfrag_row[FN], xfrag_row[FM];
@@ -748,29 +819,68 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     const int total_items = my_tiles * KT;
 
     // The block's work is one flat stream of K-slices ("items"): KT per tile, tile after
-    // tile.  Item i lives in ring slot i % STAGES.  The issue side runs STAGES-1 items ahead
-    // of the compute side and crosses tile boundaries on its own; it only needs the row
-    // pointers of the tile it is in, the compute side only the TileInfo for the epilogue.
+    // tile.  Item i lives in ring slot i % STAGES.  The issue side runs ahead of the compute
+    // side and crosses tile boundaries on its own; it only needs the row pointers of the
+    // tile it is in, the compute side only the TileInfo for the epilogue.
     TileInfo cur = locate(logical);         // tile being computed
     TileInfo nxt = cur;                     // tile after it (located one tile ahead)
     int64_t ilogical = logical;
     int ikt = 0;                            // next K-slice to issue inside the issue tile
     int issued = 0;                         // items issued so far
+    int islot = 0;                          // issued % STAGES
     int64_t ridx_next[XI];
     {
         int64_t r0[XI];
         fetch_rows(cur, r0);
         make_ptrs(cur, r0);
     }
-    auto issue_one = [&]() {
+    auto issue_next = [&]() {
         if (issued >= total_items) return;
         if (ikt == KT) {                    // the issue side enters the next tile
             make_ptrs(nxt, ridx_next);
             ikt = 0;
         }
-        issue(ikt, issued % STAGES);
-        ++ikt;
-        ++issued;
+        const int sa = islot;
+        islot = islot + 1 == STAGES ? 0 : islot + 1;
+        if (PAIR) {
+            issue(ikt, sa, islot);
+            islot = islot + 1 == STAGES ? 0 : islot + 1;
+            ikt += 2;
+            issued += 2;
+        } else {
+            issue(ikt, sa, sa);
+            ++ikt;
+            ++issued;
+        }
+    };
+    // The same pair issue cut into L parts (one row group, both halves of its 128-byte lines)
+    // so that the parts can be spread between MFMAs: a burst of VMEM instructions from all
+    // waves backs up the CU's one address path and every wave sits in its issue, unable to
+    // start MFMAs, until its own instructions are through.
+    bool part_go = false;
+    uint32_t part_a = 0, part_b = 0;
+    int64_t part_koff = 0;
+    auto issue_begin = [&]() {
+        part_go = issued < total_items;
+        if (!part_go) return;
+        if (ikt == KT) {
+            make_ptrs(nxt, ridx_next);
+            ikt = 0;
+        }
+        part_a = lds_base + islot * TL::STAGE_BYTES;
+        islot = islot + 1 == STAGES ? 0 : islot + 1;
+        part_b = lds_base + islot * TL::STAGE_BYTES;
+        islot = islot + 1 == STAGES ? 0 : islot + 1;
+        part_koff = (int64_t)ikt * 64;
+        ikt += 2;
+        issued += 2;
+    };
+    auto issue_part = [&](int j) {          // j is a compile-time constant after unrolling
+        const uint8_t* base = (j < XI ? xbase : wbase[j >= XI ? j - XI : 0]) + part_koff;
+        const uint32_t voff = j < XI ? xoff[j < XI ? j : 0] : woff[j >= XI ? j - XI : 0];
+        const uint32_t off = (j < XI ? (j * NW + wave) * 1024 : BM * 64 + ((j - XI) * NW + wave) * 1024);
+        dma16(base, voff, part_a + off);
+        dma16(base + 64, voff, part_b + off);
     };
     auto prefetch_next = [&]() {            // once per tile, early: locate the next tile and
         ilogical += nslots;                 // start fetching its source-row indices
@@ -780,13 +890,19 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         }
     };
     prefetch_next();
-    for (int j = 0; j < STAGES - 1; ++j) issue_one();
+    if (PAIR) {
+        issue_next();                       // items 0..3
+        issue_next();
+    } else {
+        for (int j = 0; j < STAGES - 1; ++j) issue_next();
+    }
 
-    // vmcnt bookkeeping.  Loads return in order, so "at most n*L operations outstanding"
-    // means every slice but the n youngest has landed; stores or other loads in the queue
-    // only make the wait longer, never shorter.
+    // vmcnt bookkeeping.  Loads return in order, so "at most n operations outstanding"
+    // means everything but the n youngest operations has landed; stores or other loads in
+    // the queue only make the wait longer, never shorter.
     int landed = -1;                        // items <= landed are complete for this wave
     int c = 0;                              // item being computed
+    int cslot = 0;                          // c % STAGES
     for (int tile_i = 0; tile_i < my_tiles; ++tile_i) {
         f32x16 acc[FN][FM];
 #pragma unroll
@@ -797,18 +913,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
         if (tile_i > 0) prefetch_next();
 
-        for (int kt = 0; kt < KT; ++kt, ++c) {
-            if (c > landed) {
-                const int younger = issued - 1 - c;
-                if (younger >= 2) wait_vmcnt<2 * L>();
-                else if (younger == 1) wait_vmcnt<L>();
-                else wait_vmcnt<0>();
-            }
-            // after this barrier every wave's share of item c is visible and every wave has
-            // finished reading item c-1, whose slot the next issue overwrites
-            __syncthreads();
-            issue_one();
-            const uint8_t* sx = smem + (c % STAGES) * TL::STAGE_BYTES;
+        auto mma_slice = [&]() {
+            const uint8_t* sx = smem + cslot * TL::STAGE_BYTES;
             const uint8_t* sw = sx + BM * 64;
             if (!FP8) {
 #pragma unroll
@@ -848,11 +954,130 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                     for (int fm = 0; fm < FM; ++fm)
                         acc[fn][fm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0, 0, 0, 0);
             }
+            ++c;
+            cslot = cslot + 1 == STAGES ? 0 : cslot + 1;
+        };
+
+        if constexpr (PAIR && !FP8) {
+            // Software pipeline over "blocks" (half a K-slice: one 16-byte chunk per row and
+            // lane half, 8 MFMAs): the fragments of block b+1 are read while block b
+            // multiplies.  Two barriers per pair of items c, c+1:
+            //   B  after the last read of item c      -> its slot and the one of c-1 are refilled
+            //   A' before the first read of item c+2  -> pair (c+2, c+3) has landed everywhere
+            // Raw s_barrier (no fence): LDS reads of slots that stay valid may be in flight
+            // across a barrier; the asm statements keep the compiler from moving LDS reads
+            // over them.
+            bf16x8 wfa[FN], xfa[FM], wfb[FN], xfb[FM];
+            auto load_block = [&](bf16x8 (&wf)[FN], bf16x8 (&xf)[FM], int slot_i, int sub) {
+                const uint8_t* sx = smem + slot_i * TL::STAGE_BYTES;
+                const uint8_t* sw = sx + BM * 64;
+                const int chunk = 2 * sub + khalf;
+#pragma unroll
+                for (int fn = 0; fn < FN; ++fn)
+                    wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
+#pragma unroll
+                for (int fm = 0; fm < FM; ++fm)
+                    xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
+            };
+            // the 8 MFMAs of a block; when `phase` names this wave's half of the block (waves w
+            // and w + NW/2 share a SIMD) the L parts of the pair being issued go out between
+            // them.  The two waves of a SIMD issue in different blocks, so that while one
+            // sits in its VMEM issue the other keeps the MFMA pipe busy.
+            const int half = wave >= NW / 2 ? 1 : 0;
+            auto mma_block = [&](const bf16x8 (&wf)[FN], const bf16x8 (&xf)[FM], int phase) {
+                constexpr int NM = FN * FM, EVERY = NM / L;
+                const bool mine = part_go && phase == half;
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    const int fn = m / FM, fm = m % FM;
+                    acc[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0);
+                    if (phase >= 0 && (m + 1) % EVERY == 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (mine) issue_part((m + 1) / EVERY - 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            };
+            auto barrier = [&]() {
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            };
+            if (tile_i == 0) {              // pair 0 has landed everywhere
+                if (issued >= 4) wait_vmcnt<2 * L>();
+                else wait_vmcnt<0>();
+                barrier();
+            }
+            // sched_barrier(0) pins the order "reads of the next block, then the MFMAs of this
+            // one"; left alone the scheduler sinks the reads to just before their first use.
+            load_block(wfa, xfa, cslot, 0);
+            for (int kt = 0; kt < KT; kt += 2) {
+                const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
+                const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
+                load_block(wfb, xfb, cslot, 1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(wfa, xfa, -1);
+                __builtin_amdgcn_sched_barrier(0);
+                load_block(wfa, xfa, s1, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(wfb, xfb, -1);
+                __builtin_amdgcn_sched_barrier(0);
+                barrier();                  // B
+                issue_begin();              // pair (c+4, c+5); its instructions go out below
+                load_block(wfb, xfb, s1, 1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(wfa, xfa, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                // pair (c+2, c+3) is older than the 2L instructions the first half just issued
+                if (part_go && half == 0) wait_vmcnt<2 * L>();
+                else wait_vmcnt<0>();
+                barrier();                  // A'
+                if (kt + 2 < KT) load_block(wfa, xfa, s2, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(wfb, xfb, 1);
+                __builtin_amdgcn_sched_barrier(0);
+                c += 2;
+                cslot = s2;
+            }
+        } else if constexpr (PAIR) {
+            // Pair q = items 2q, 2q+1.  It is issued at the start of odd step 2q-3, into the
+            // slots of items 2q-5 and 2q-4 whose last readers passed that step's barrier, and
+            // is needed at even step 2q, when at most one younger pair is outstanding.
+            for (int kt = 0; kt < KT; kt += 2) {
+                if (c > landed) {
+                    if (issued - c >= 4) wait_vmcnt<2 * L>();
+                    else wait_vmcnt<0>();
+                }
+                __syncthreads();            // item c and c+1 visible from every wave
+                mma_slice();
+                __syncthreads();            // every wave is done with item c-1 (now c-2) ...
+                issue_next();               // ... whose slot, with the one before it, is refilled
+                mma_slice();
+            }
+            // all but the youngest pair have landed after this wait, so the first pair of the
+            // next tile needs no vmcnt wait and the epilogue's stores drain behind it
+            wait_vmcnt<2 * L>();
+            landed = issued - 3;
+        } else {
+            for (int kt = 0; kt < KT; ++kt) {
+                if (c > landed) {
+                    const int younger = issued - 1 - c;
+                    if (younger >= 2) wait_vmcnt<2 * L>();
+                    else if (younger == 1) wait_vmcnt<L>();
+                    else wait_vmcnt<0>();
+                }
+                // after this barrier every wave's share of item c is visible and every wave
+                // has finished reading item c-1, whose slot the next issue overwrites
+                __syncthreads();
+                issue_next();
+                mma_slice();
+            }
+            // All but the youngest issued slice have landed after this wait, so the first
+            // slices of the next tile need no vmcnt wait and the epilogue's stores drain
+            // behind them.
+            wait_vmcnt<L>();
+            landed = issued - 2;
         }
-        // All but the youngest issued slice have landed after this wait, so the first slices
-        // of the next tile need no vmcnt wait and the epilogue's stores drain behind them.
-        wait_vmcnt<L>();
-        landed = issued - 2;
         const TileInfo done = cur;
         cur = nxt;      // valid when another tile follows (nxt was located at this tile's start)
 
@@ -865,7 +1090,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 // ------------------------------------------------------------------- host side
 typedef TileCfg<256, 256, 2, 4> TileBig;        // 8 waves, wave tile 128 x 64
 typedef TileCfg<64, 256, 1, 4> TileSmall;       // 4 waves, wave tile 64 x 64
-typedef RingCfg<256, 256, 2, 4, 4> TileRing;    // 8 waves, wave tile 128 x 64, 4-slot ring
+typedef RingCfg<256, 256, 2, 4, 0> TileRing4;   // 8 waves, wave tile 128 x 64, 4-slot ring, LDS tables
+typedef RingCfg<256, 256, 2, 4, 1> TileRing5;   // 5-slot ring, paired slices, E <= 64
+typedef RingCfg<256, 256, 2, 4, 4> TileRing5W;  // 5-slot ring, paired slices, E <= 256
 
 enum GemmKernelSel { kSelRing = 0, kSelStagedBig = 1, kSelStagedSmall = 2, kSelGeneric = 3 };
 
@@ -897,10 +1124,10 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
 }
 
 int compute_units();   // CUs of the current device (gemm_api.hip)
+int lds_per_block();   // largest LDS allocation of one block on the current device (gemm_api.hip)
 
-template <bool FP8, int EPI>
-int launch_ring(GemmParams p, hipStream_t stream) {
-    typedef TileRing TL;
+template <typename TL, bool FP8, int EPI>
+int launch_ring_cfg(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
     auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI>;
@@ -912,6 +1139,18 @@ int launch_ring(GemmParams p, hipStream_t stream) {
     if (grid < kNumXcd) grid = kNumXcd;
     kern<<<(unsigned)grid, TL::NT, TL::LDS_BYTES, stream>>>(p);
     return check_launch("fmoe_grouped_gemm");
+}
+
+// The 5-slot ring needs every byte of a 160 KB LDS, an even number of K-slices per tile,
+// row numbers that fit 32 bits and few enough experts for the register tables.
+template <bool FP8, int EPI>
+int launch_ring(const GemmParams& p, hipStream_t stream) {
+    const int slices = p.K / (FP8 ? 64 : 32);
+    const bool pair_ok = slices % 2 == 0 && slices >= 4 && p.total_rows < ((int64_t)1 << 31) &&
+                         lds_per_block() >= TileRing5::LDS_BYTES;
+    if (pair_ok && p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI>(p, stream);
+    if (pair_ok && p.E <= TileRing5W::kMaxExperts) return launch_ring_cfg<TileRing5W, FP8, EPI>(p, stream);
+    return launch_ring_cfg<TileRing4, FP8, EPI>(p, stream);
 }
 
 template <int DT, int EPI, bool A_SILU>
