@@ -33,6 +33,8 @@
 
 #include "common.h"
 
+#include <type_traits>
+
 namespace fmoe {
 
 typedef __attribute__((ext_vector_type(2))) float f32x2;
@@ -829,6 +831,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int issued = 0;                         // items issued so far
     int islot = 0;                          // issued % STAGES
     int64_t ridx_next[XI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) ridx_next[i] = 0;
     {
         int64_t r0[XI];
         fetch_rows(cur, r0);
@@ -857,24 +861,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     // so that the parts can be spread between MFMAs: a burst of VMEM instructions from all
     // waves backs up the CU's one address path and every wave sits in its issue, unable to
     // start MFMAs, until its own instructions are through.
-    bool part_go = false;
     uint32_t part_a = 0, part_b = 0;
     int64_t part_koff = 0;
-    auto issue_begin = [&]() {
-        part_go = issued < total_items;
-        if (!part_go) return;
-        if (ikt == KT) {
-            make_ptrs(nxt, ridx_next);
-            ikt = 0;
-        }
-        part_a = lds_base + islot * TL::STAGE_BYTES;
-        islot = islot + 1 == STAGES ? 0 : islot + 1;
-        part_b = lds_base + islot * TL::STAGE_BYTES;
-        islot = islot + 1 == STAGES ? 0 : islot + 1;
-        part_koff = (int64_t)ikt * 64;
-        ikt += 2;
-        issued += 2;
-    };
     auto issue_part = [&](int j) {          // j is a compile-time constant after unrolling
         const uint8_t* base = (j < XI ? xbase : wbase[j >= XI ? j - XI : 0]) + part_koff;
         const uint32_t voff = j < XI ? xoff[j < XI ? j : 0] : woff[j >= XI ? j - XI : 0];
@@ -903,6 +891,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int landed = -1;                        // items <= landed are complete for this wave
     int c = 0;                              // item being computed
     int cslot = 0;                          // c % STAGES
+    bf16x8 wfa[FN], xfa[FM], wfb[FN], xfb[FM];   // fragment double buffer of the pipelined loop
     for (int tile_i = 0; tile_i < my_tiles; ++tile_i) {
         f32x16 acc[FN][FM];
 #pragma unroll
@@ -961,13 +950,15 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         if constexpr (PAIR && !FP8) {
             // Software pipeline over "blocks" (half a K-slice: one 16-byte chunk per row and
             // lane half, 8 MFMAs): the fragments of block b+1 are read while block b
-            // multiplies.  Two barriers per pair of items c, c+1:
+            // multiplies.  Two barriers per pair of items c, c+1 (a "double step"):
             //   B  after the last read of item c      -> its slot and the one of c-1 are refilled
             //   A' before the first read of item c+2  -> pair (c+2, c+3) has landed everywhere
             // Raw s_barrier (no fence): LDS reads of slots that stay valid may be in flight
             // across a barrier; the asm statements keep the compiler from moving LDS reads
-            // over them.
-            bf16x8 wfa[FN], xfa[FM], wfb[FN], xfb[FM];
+            // over them.  The steady state is straight-line code: the issue side always has
+            // something to fetch (past the end of the block's stream it re-reads the last
+            // tile's rows into slots nobody looks at), and everything that depends on the
+            // wave's half is a template parameter.
             auto load_block = [&](bf16x8 (&wf)[FN], bf16x8 (&xf)[FM], int slot_i, int sub) {
                 const uint8_t* sx = smem + slot_i * TL::STAGE_BYTES;
                 const uint8_t* sw = sx + BM * 64;
@@ -979,21 +970,19 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 for (int fm = 0; fm < FM; ++fm)
                     xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
             };
-            // the 8 MFMAs of a block; when `phase` names this wave's half of the block (waves w
-            // and w + NW/2 share a SIMD) the L parts of the pair being issued go out between
-            // them.  The two waves of a SIMD issue in different blocks, so that while one
-            // sits in its VMEM issue the other keeps the MFMA pipe busy.
-            const int half = wave >= NW / 2 ? 1 : 0;
-            auto mma_block = [&](const bf16x8 (&wf)[FN], const bf16x8 (&xf)[FM], int phase) {
+            // the 8 MFMAs of a block, with the L parts of the pair being issued between them
+            // when DMA is set.  The two waves of a SIMD (w and w + NW/2) issue in different
+            // blocks, so that while one sits in its VMEM issue the other feeds the MFMA pipe.
+            auto mma_block = [&](const bf16x8 (&wf)[FN], const bf16x8 (&xf)[FM], auto dma_c) {
+                constexpr bool DMA = decltype(dma_c)::value;
                 constexpr int NM = FN * FM, EVERY = NM / L;
-                const bool mine = part_go && phase == half;
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int fn = m / FM, fm = m % FM;
                     acc[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0);
-                    if (phase >= 0 && (m + 1) % EVERY == 0) {
+                    if (DMA && (m + 1) % EVERY == 0) {
                         __builtin_amdgcn_sched_barrier(0);
-                        if (mine) issue_part((m + 1) / EVERY - 1);
+                        issue_part((m + 1) / EVERY - 1);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -1003,42 +992,57 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             };
-            if (tile_i == 0) {              // pair 0 has landed everywhere
-                if (issued >= 4) wait_vmcnt<2 * L>();
-                else wait_vmcnt<0>();
-                barrier();
-            }
             // sched_barrier(0) pins the order "reads of the next block, then the MFMAs of this
             // one"; left alone the scheduler sinks the reads to just before their first use.
-            load_block(wfa, xfa, cslot, 0);
-            for (int kt = 0; kt < KT; kt += 2) {
+            auto double_step = [&](auto half_c, auto last_c) {
+                constexpr int HALF = decltype(half_c)::value;
+                constexpr bool LAST = decltype(last_c)::value;   // last of the tile: no fragments kept over the epilogue
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
                 const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
                 load_block(wfb, xfb, cslot, 1);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(wfa, xfa, -1);
+                mma_block(wfa, xfa, std::false_type{});
                 __builtin_amdgcn_sched_barrier(0);
                 load_block(wfa, xfa, s1, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(wfb, xfb, -1);
+                mma_block(wfb, xfb, std::false_type{});
                 __builtin_amdgcn_sched_barrier(0);
                 barrier();                  // B
-                issue_begin();              // pair (c+4, c+5); its instructions go out below
+                part_a = lds_base + islot * TL::STAGE_BYTES;    // pair (c+4, c+5)
+                islot = islot + 1 == STAGES ? 0 : islot + 1;
+                part_b = lds_base + islot * TL::STAGE_BYTES;
+                islot = islot + 1 == STAGES ? 0 : islot + 1;
+                part_koff = (int64_t)ikt * 64;
+                ikt += 2;
                 load_block(wfb, xfb, s1, 1);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(wfa, xfa, 0);
+                mma_block(wfa, xfa, std::integral_constant<bool, HALF == 0>{});
                 __builtin_amdgcn_sched_barrier(0);
                 // pair (c+2, c+3) is older than the 2L instructions the first half just issued
-                if (part_go && half == 0) wait_vmcnt<2 * L>();
+                if (HALF == 0) wait_vmcnt<2 * L>();
                 else wait_vmcnt<0>();
                 barrier();                  // A'
-                if (kt + 2 < KT) load_block(wfa, xfa, s2, 0);
+                if (!LAST) load_block(wfa, xfa, s2, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(wfb, xfb, 1);
+                mma_block(wfb, xfb, std::integral_constant<bool, HALF == 1>{});
                 __builtin_amdgcn_sched_barrier(0);
-                c += 2;
                 cslot = s2;
+            };
+            // the issue side runs 4 items ahead: it enters the next tile 4 items before the end
+            auto tile_steps = [&](auto half_c) {
+                for (int kt = 0; kt < KT - 4; kt += 2) double_step(half_c, std::false_type{});
+                make_ptrs(nxt, ridx_next);
+                ikt = 0;
+                double_step(half_c, std::false_type{});
+                double_step(half_c, std::true_type{});
+            };
+            if (tile_i == 0) {              // pair 0 has landed everywhere
+                wait_vmcnt<2 * L>();
+                barrier();
             }
+            load_block(wfa, xfa, cslot, 0);
+            if (wave < NW / 2) tile_steps(std::integral_constant<int, 0>{});
+            else tile_steps(std::integral_constant<int, 1>{});
         } else if constexpr (PAIR) {
             // Pair q = items 2q, 2q+1.  It is issued at the start of odd step 2q-3, into the
             // slots of items 2q-5 and 2q-4 whose last readers passed that step's barrier, and
@@ -1084,6 +1088,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         gemm_epilogue<FM, FN, TM, TN, FP8, EPI>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                 done.rows_valid, wm, wn, lane);
     }
+    wait_vmcnt<0>();    // nothing may still be on its way into this block's LDS when it ends
 }
 
 
