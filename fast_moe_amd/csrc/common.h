@@ -52,7 +52,10 @@ __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)
 
 // SiLU from the hardware exp / reciprocal (about 2 ulp in fp32): for values that
 // are rounded to bf16 right afterwards.
-__device__ __forceinline__ float fast_silu_f32(float x) { return __fdividef(x, 1.0f + __expf(-x)); }
+__device__ __forceinline__ float fast_silu_f32(float x) {
+    // v_exp_f32 and v_rcp_f32 only: a true division costs ten more VALU instructions
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896341f));
+}
 
 __device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 
