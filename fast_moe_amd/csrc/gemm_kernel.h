@@ -892,6 +892,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int c = 0;                              // item being computed
     int cslot = 0;                          // c % STAGES
     bf16x8 wfa[FN], xfa[FM], wfb[FN], xfb[FM];   // fragment double buffer of the pipelined loop
+    i32x8 qwa[FN], qwb[FN], qx0[FM / 2], qx1[FM / 2];   // the same for e4m3 fragments
     for (int tile_i = 0; tile_i < my_tiles; ++tile_i) {
         f32x16 acc[FN][FM];
 #pragma unroll
@@ -1044,24 +1045,99 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             if (wave < NW / 2) tile_steps(std::integral_constant<int, 0>{});
             else tile_steps(std::integral_constant<int, 1>{});
         } else if constexpr (PAIR) {
-            // Pair q = items 2q, 2q+1.  It is issued at the start of odd step 2q-3, into the
-            // slots of items 2q-5 and 2q-4 whose last readers passed that step's barrier, and
-            // is needed at even step 2q, when at most one younger pair is outstanding.
-            for (int kt = 0; kt < KT; kt += 2) {
-                if (c > landed) {
-                    if (issued - c >= 4) wait_vmcnt<2 * L>();
-                    else wait_vmcnt<0>();
+            // e4m3: the same double step; an item is one 32x32x64 MFMA deep, so its two blocks
+            // split the activation fragments instead of K: block 0 reads both weight
+            // fragments and activation fragments 0..FM/2-1, block 1 the other activation
+            // fragments and reuses the weights.
+            constexpr int HM = FM / 2;
+            auto load_frag = [&](const uint8_t* base, int row) -> i32x8 {
+                const int chunk = 2 * khalf;
+                const u32x4 lo = *reinterpret_cast<const u32x4*>(base + lds_off64(row, chunk));
+                const u32x4 hi = *reinterpret_cast<const u32x4*>(base + lds_off64(row, chunk + 1));
+                return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            };
+            auto load_w_x0 = [&](i32x8 (&wf)[FN], i32x8 (&xh)[HM], int slot_i) {
+                const uint8_t* sx = smem + slot_i * TL::STAGE_BYTES;
+#pragma unroll
+                for (int fn = 0; fn < FN; ++fn) wf[fn] = load_frag(sx + BM * 64, wfrag_row[fn]);
+#pragma unroll
+                for (int fm = 0; fm < HM; ++fm) xh[fm] = load_frag(sx, xfrag_row[fm]);
+            };
+            auto load_x1 = [&](i32x8 (&xh)[HM], int slot_i) {
+                const uint8_t* sx = smem + slot_i * TL::STAGE_BYTES;
+#pragma unroll
+                for (int fm = 0; fm < HM; ++fm) xh[fm] = load_frag(sx, xfrag_row[HM + fm]);
+            };
+            auto mma_block = [&](const i32x8 (&wf)[FN], const i32x8 (&xh)[HM], int fm0, auto dma_c) {
+                constexpr bool DMA = decltype(dma_c)::value;
+                constexpr int NM = FN * HM;
+                static_assert(NM % L == 0 || L % NM == 0, "DMA parts must spread evenly over the MFMAs");
+                constexpr int PER = L >= NM ? L / NM : 1, EVERY = L >= NM ? 1 : NM / L;
+#pragma unroll
+                for (int m = 0; m < NM; ++m) {
+                    const int fn = m / HM, fm = m % HM;
+                    acc[fn][fm0 + fm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                        wf[fn], xh[fm], acc[fn][fm0 + fm], 0, 0, 0, 0, 0, 0);
+                    if (DMA && (m + 1) % EVERY == 0) {
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int q = 0; q < PER; ++q) issue_part(((m + 1) / EVERY - 1) * PER + q);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
-                __syncthreads();            // item c and c+1 visible from every wave
-                mma_slice();
-                __syncthreads();            // every wave is done with item c-1 (now c-2) ...
-                issue_next();               // ... whose slot, with the one before it, is refilled
-                mma_slice();
+            };
+            auto barrier = [&]() {
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            };
+            auto double_step = [&](auto half_c, auto last_c) {
+                constexpr int HALF = decltype(half_c)::value;
+                constexpr bool LAST = decltype(last_c)::value;
+                const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
+                const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
+                load_x1(qx1, cslot);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(qwa, qx0, 0, std::false_type{});
+                __builtin_amdgcn_sched_barrier(0);
+                load_w_x0(qwb, qx0, s1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(qwa, qx1, HM, std::false_type{});
+                __builtin_amdgcn_sched_barrier(0);
+                barrier();                  // B
+                part_a = lds_base + islot * TL::STAGE_BYTES;    // pair (c+4, c+5)
+                islot = islot + 1 == STAGES ? 0 : islot + 1;
+                part_b = lds_base + islot * TL::STAGE_BYTES;
+                islot = islot + 1 == STAGES ? 0 : islot + 1;
+                part_koff = (int64_t)ikt * 64;
+                ikt += 2;
+                load_x1(qx1, s1);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(qwb, qx0, 0, std::integral_constant<bool, HALF == 0>{});
+                __builtin_amdgcn_sched_barrier(0);
+                if (HALF == 0) wait_vmcnt<2 * L>();
+                else wait_vmcnt<0>();
+                barrier();                  // A'
+                if (!LAST) load_w_x0(qwa, qx0, s2);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_block(qwb, qx1, HM, std::integral_constant<bool, HALF == 1>{});
+                __builtin_amdgcn_sched_barrier(0);
+                cslot = s2;
+            };
+            auto tile_steps = [&](auto half_c) {
+                for (int kt = 0; kt < KT - 4; kt += 2) double_step(half_c, std::false_type{});
+                make_ptrs(nxt, ridx_next);
+                ikt = 0;
+                double_step(half_c, std::false_type{});
+                double_step(half_c, std::true_type{});
+            };
+            if (tile_i == 0) {              // pair 0 has landed everywhere
+                wait_vmcnt<2 * L>();
+                barrier();
             }
-            // all but the youngest pair have landed after this wait, so the first pair of the
-            // next tile needs no vmcnt wait and the epilogue's stores drain behind it
-            wait_vmcnt<2 * L>();
-            landed = issued - 3;
+            load_w_x0(qwa, qx0, cslot);
+            if (wave < NW / 2) tile_steps(std::integral_constant<int, 0>{});
+            else tile_steps(std::integral_constant<int, 1>{});
         } else {
             for (int kt = 0; kt < KT; ++kt) {
                 if (c > landed) {
