@@ -6,9 +6,12 @@
 //
 //   grouped_gemm_ring_kernel   the fast path.  Persistent (one block per CU), 256 x 256 tiles,
 //       8 wavefronts.  Operand K-slices of 64 bytes per row travel global -> LDS with
-//       global_load_lds_dwordx4 (no VGPR staging) into a 4-slot ring, three slices in flight
-//       per CU; the ring runs across tile boundaries, so the loads of the next tile are
-//       already under way while the current tile's epilogue stores drain.
+//       global_load_lds_dwordx4 (no VGPR staging) into a ring of 32 KB slots; the ring runs
+//       across tile boundaries, so the loads of the next tile are already under way while
+//       the current tile's epilogue stores drain.  With few experts the ring takes all of
+//       LDS (5 slots), slices are fetched in pairs as full 128-byte lines and the K loop is
+//       a software pipeline of 8-MFMA blocks (see RingCfg); otherwise 4 slots, one slice at
+//       a time, schedule tables in LDS.
 //   grouped_gemm_kernel        register-staged, double-buffered LDS; serves everything the
 //       ring kernel does not: arbitrary B strides and K / N tails (element loads), SiLU
 //       applied to A on load, and short 64-row tiles for experts with a handful of rows.
