@@ -11,6 +11,7 @@ tensors of any strides, except ``silu_jagged_bmm_fp8`` which keeps the
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -36,6 +37,59 @@ def quantize_expert_weights(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.T
     quantisation kernels/pytorch/moe_fp8.py:111 redoes on every call; do it once per weight update."""
     q, s = ops.quant_rows_fp8(weight.permute(0, 2, 1))     # [E, N, K] contiguous
     return q.permute(0, 2, 1), s
+
+
+class _WeightQuantCache:
+    """(fp8 bytes, scales) of expert weights, kept until the weight changes.
+
+    The reference quantises the weights inside every fp8 operator call
+    (kernels/pytorch/moe_fp8.py:111, kernels/triton/triton_moe_fp8.py:1157, 1423): 3 bytes of
+    HBM traffic per weight element per forward.  An entry is keyed by the tensor that owns
+    the storage (the parameter behind a ``permute``/``to`` view, held weakly) and by the
+    view's geometry; it is dropped when the owner's in-place version counter moves (an
+    optimizer step, ``copy_``, ``load_state_dict``) or the owner dies.  Out-of-place
+    replacement (``layer.w = new``) makes a new owner and therefore a new entry.
+    """
+
+    def __init__(self, max_entries: int = 32) -> None:
+        self._entries: "dict[int, tuple]" = {}
+        self._max = max_entries
+        self.hits = 0
+        self.misses = 0
+
+    @staticmethod
+    def _owner(weight: torch.Tensor) -> torch.Tensor:
+        return weight._base if weight._base is not None else weight
+
+    def get(self, weight: torch.Tensor, quantize) -> Tuple[torch.Tensor, torch.Tensor]:
+        owner = self._owner(weight)
+        geom = (weight.data_ptr(), tuple(weight.shape), tuple(weight.stride()), weight.dtype, str(weight.device))
+        key = id(owner)
+        hit = self._entries.get(key)
+        if hit is not None:
+            ref, version, cached_geom, value = hit
+            if ref() is owner and version == owner._version and cached_geom == geom:
+                self.hits += 1
+                return value
+        self.misses += 1
+        value = quantize(weight)
+        if len(self._entries) >= self._max:
+            dead = [k for k, (r, *_rest) in self._entries.items() if r() is None]
+            for k in dead or list(self._entries)[:1]:
+                self._entries.pop(k, None)
+        self._entries[key] = (weakref.ref(owner), owner._version, geom, value)
+        return value
+
+    def clear(self) -> None:
+        self._entries.clear()
+
+
+weight_quant_cache = _WeightQuantCache()
+
+
+def cached_quantize_expert_weights(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``quantize_expert_weights`` through ``weight_quant_cache``."""
+    return weight_quant_cache.get(weight, quantize_expert_weights)
 
 
 def silu_jagged_fp8(
@@ -102,7 +156,7 @@ def silu_jagged_bmm_combine_fp8(
     assert index.shape[0] == L * K == jagged.shape[0]
     ops._forward_only("silu_jagged_bmm_combine_fp8", jagged, weight, bias, gating_scores)
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
-    qw, sw = quantize_expert_weights(weight)
+    qw, sw = cached_quantize_expert_weights(weight)
     bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias, a_scale=sa,
                                b_scale=sw, epilogue=EPI_NONE)
     return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
@@ -129,7 +183,7 @@ def index_select_jagged_bmm(
                                 index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
     assert jagged.dtype == weight.dtype and (bias is None or jagged.dtype == bias.dtype)
     qa, sa = ops.quant_rows_fp8(jagged)
-    qw, sw = quantize_expert_weights(weight)
+    qw, sw = cached_quantize_expert_weights(weight)
     return ops.grouped_gemm(offsets, qa, qw, total_rows=index.numel(), row_index=index,
                             index_div=index.shape[-1], bias=bias, a_scale=sa, b_scale=sw,
                             epilogue=EPI_NONE)

@@ -130,3 +130,33 @@ def test_state_dict_layout_matches_reference_names():
                        "_experts_w", "_experts_bias"}
     assert tuple(sd["_experts_hidden_w"].shape) == (4, 32, 16)
     assert tuple(sd["_experts_w"].shape) == (4, 8, 32)
+
+
+def test_weight_quant_cache_hits_and_invalidation():
+    """The cache logic of moe_fp8 on CPU tensors with a stand-in quantiser (no GPU work)."""
+    import torch
+    from fast_moe_amd.kernels.moe_fp8 import _WeightQuantCache
+    cache = _WeightQuantCache(max_entries=4)
+    calls = []
+
+    def quantize(w):
+        calls.append(w.data_ptr())
+        return (w.detach().clone(), w.abs().amax(1))
+
+    param = torch.nn.Parameter(torch.randn(3, 8, 4))
+    view = lambda: param.permute(0, 2, 1)
+    a = cache.get(view(), quantize)
+    b = cache.get(view(), quantize)                       # a fresh view object of the same owner
+    assert len(calls) == 1 and a[0] is b[0] and (cache.hits, cache.misses) == (1, 1)
+    with torch.no_grad():
+        param.mul_(2.0)                                   # in-place update: version counter moves
+    c = cache.get(view(), quantize)
+    assert len(calls) == 2 and torch.equal(c[0], view())
+    d = cache.get(param[:2].permute(0, 2, 1), quantize)   # another geometry of the same owner
+    assert len(calls) == 3 and d[0].shape[0] == 2
+    other = torch.randn(3, 4, 8)
+    cache.get(other, quantize)
+    del other
+    for _ in range(6):                                    # dead owners are evicted, the table stays bounded
+        cache.get(torch.randn(3, 4, 8), quantize)
+    assert len(cache._entries) <= 4

@@ -140,3 +140,24 @@ def test_silu_quant_and_weight_quant():
     q3_ref, s3_ref = o_fp8.rowwise_quant_fp8(w.permute(0, 2, 1).float().numpy(), "bf16")
     assert np.array_equal(q3.permute(0, 2, 1).contiguous().view(torch.uint8).cpu().numpy(), q3_ref)
     assert np.array_equal(s3.cpu().numpy(), s3_ref)
+
+
+def test_fp8_operator_reuses_cached_weight_quantisation():
+    """index_select_jagged_bmm(fp8=True) quantises a weight once and again only after an update."""
+    from fast_moe_amd.kernels import moe_fp8
+    from helpers import make_routing, randn
+    r = make_routing(512, 8, 2, seed=5)
+    x = randn((512, 128), 1).cuda()
+    w = (randn((8, 128, 96), 2) * 128 ** -0.5).cuda()
+    off, idx = r["offsets"].cuda(), r["index"].cuda()
+    cache = moe_fp8.weight_quant_cache
+    cache.clear()
+    h0, m0 = cache.hits, cache.misses
+    with torch.no_grad():
+        y1 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
+        y2 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
+        assert (cache.hits - h0, cache.misses - m0) == (1, 1) and torch.equal(y1, y2)
+        w.mul_(2.0)
+        y3 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
+    assert cache.misses - m0 == 2
+    torch.testing.assert_close(y3.float(), 2 * y1.float(), rtol=0, atol=0)   # a power of two: exact
