@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(HERE, "libfastmoe_hip.so")
 OBJ_DIR = os.path.join(CSRC, "build")
 
 SOURCES = ["core.hip", "routing.hip", "quant.hip", "combine.hip", "gemm_api.hip", "gemm_bf16.hip",
-           "gemm_fp8.hip", "gemm_f32.hip"]
+           "gemm_fp8.hip", "gemm_f32.hip", "backward.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

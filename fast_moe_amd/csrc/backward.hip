@@ -1,0 +1,258 @@
+// Backward helpers of the MoE path: operand transposition for the weight-gradient GEMM,
+// bias gradients, SwiGLU / SiLU backward and the backward of the weighted merge.
+#include "common.h"
+
+namespace fmoe {
+namespace {
+
+template <typename T> struct Val;
+template <> struct Val<uint16_t> {
+    __device__ static float load(const uint16_t* p) { return bf16_bits_to_f32(*p); }
+    __device__ static void store(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
+    __device__ static float round(float v) { return round_bf16(v); }
+};
+template <> struct Val<float> {
+    __device__ static float load(const float* p) { return *p; }
+    __device__ static void store(float* p, float v) { *p = v; }
+    __device__ static float round(float v) { return v; }
+};
+
+// 64 (padded rows) x 64 (columns) tile: every thread column finds the expert that owns its
+// padded row by binary search in pad_offsets, reads the source row it maps to (or zero for
+// padding) and the tile is written transposed through LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void jagged_transpose_kernel(
+    const T* __restrict__ src, int64_t src_rows, int64_t cols, int64_t src_stride,
+    const int64_t* __restrict__ row_index, int index_div, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ pad_offsets, int E, T* __restrict__ dst, int64_t dst_stride,
+    int64_t dst_cols, int apply_silu) {
+    __shared__ T tile[64][64 + 2];
+    __shared__ int64_t s_src[64];
+    const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    if (threadIdx.x < 64) {
+        const int64_t pcol = p0 + threadIdx.x;
+        int64_t srow = -1;
+        if (pcol < pad_offsets[E]) {
+            int lo = 0, hi = E;               // largest e with pad_offsets[e] <= pcol
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (pad_offsets[mid] <= pcol) lo = mid; else hi = mid;
+            }
+            const int64_t j = pcol - pad_offsets[lo];
+            const int64_t len = offsets[lo + 1] - offsets[lo];
+            if (j >= 0 && j < len) {
+                int64_t r = offsets[lo] + j;
+                if (row_index) r = row_index[r] / index_div;
+                if (r >= 0 && r < src_rows) srow = r;
+            }
+        }
+        s_src[threadIdx.x] = srow;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const int64_t r = s_src[i], c = c0 + tx;
+        T v = 0;
+        if (r >= 0 && c < cols) {
+            v = src[r * src_stride + c];
+            if (apply_silu) {
+                float f = Val<T>::load(&v);
+                Val<T>::store(&v, silu_f32(f));
+            }
+        }
+        tile[i][tx] = v;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const int64_t c = c0 + i, pcol = p0 + tx;
+        if (c < cols && pcol < dst_cols) dst[c * dst_stride + pcol] = tile[tx][i];
+    }
+}
+
+// one block per (expert, 64 columns): 4 row lanes add every 4th row, then a fixed-order tree
+template <typename T>
+__global__ __launch_bounds__(256) void segment_colsum_kernel(const T* __restrict__ src, int64_t total_rows,
+                                                             int64_t cols, int64_t stride,
+                                                             const int64_t* __restrict__ offsets,
+                                                             T* __restrict__ out) {
+    __shared__ float part[4][64];
+    const int e = blockIdx.y;
+    const int64_t c = (int64_t)blockIdx.x * 64 + (threadIdx.x & 63);
+    const int ty = threadIdx.x >> 6;
+    int64_t lo = offsets[e], hi = offsets[e + 1];
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > total_rows ? total_rows : hi;
+    float acc = 0.0f;
+    if (c < cols)
+        for (int64_t r = lo + ty; r < hi; r += 4) acc += Val<T>::load(src + r * stride + c);
+    part[ty][threadIdx.x & 63] = acc;
+    __syncthreads();
+    if (ty == 0 && c < cols) {
+        const int x = threadIdx.x;
+        Val<T>::store(out + (int64_t)e * cols + c, (part[0][x] + part[1][x]) + (part[2][x] + part[3][x]));
+    }
+}
+
+__device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ g, const T* __restrict__ u,
+                                                         const T* __restrict__ dh, T* __restrict__ dg,
+                                                         T* __restrict__ du, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float gv = Val<T>::load(g + i), d = Val<T>::load(dh + i);
+    const float s = sigmoid_f32(gv);
+    const float dsilu = s * (1.0f + gv * (1.0f - s));
+    if (GATED) {
+        const float uv = Val<T>::load(u + i);
+        Val<T>::store(du + i, d * Val<T>::round(gv * s));
+        Val<T>::store(dg + i, Val<T>::round(d * uv) * dsilu);
+    } else {
+        Val<T>::store(dg + i, d * dsilu);
+    }
+}
+
+struct GateArgs {
+    const void* ptr;
+    int64_t cols, stride_row, stride_col;
+    const int64_t* index;
+    int64_t numel;
+};
+
+// one wavefront per routed row
+template <typename T, typename TG>
+__global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ value,
+                                                          int64_t T_tokens, int64_t R, int64_t D,
+                                                          int64_t value_stride,
+                                                          const int64_t* __restrict__ token_index,
+                                                          GateArgs gate, T* __restrict__ d_value,
+                                                          float* __restrict__ d_gates) {
+    const int lane = lane_id();
+    const int64_t r = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
+    if (r >= R) return;
+    int64_t t = token_index[r];
+    const bool ok = t >= 0 && t < T_tokens;
+    if (!ok) t = 0;
+    const int64_t flat = gate.index ? gate.index[r] : r;
+    float w = 1.0f;
+    const bool flat_ok = (uint64_t)flat < (uint64_t)gate.numel;
+    if (gate.ptr) {
+        w = 0.0f;
+        if (flat_ok) {
+            const int64_t gr = flat / gate.cols, gc = flat - gr * gate.cols;
+            w = Val<TG>::load((const TG*)gate.ptr + gr * gate.stride_row + gc * gate.stride_col);
+        }
+    }
+    float dot = 0.0f;
+    for (int64_t c = lane; c < D; c += kWave) {
+        const float d = ok ? Val<T>::load(dy + t * D + c) : 0.0f;
+        Val<T>::store(d_value + r * D + c, d * w);
+        if (d_gates) dot += Val<T>::round(Val<T>::load(value + r * value_stride + c) * d);
+    }
+    if (d_gates) {
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) dot += __shfl_xor(dot, o, kWave);
+        if (lane == 0 && flat_ok) d_gates[flat] = dot;
+    }
+}
+
+}  // namespace
+}  // namespace fmoe
+
+using namespace fmoe;
+
+extern "C" int fmoe_jagged_transpose(const void* src, int dtype, int64_t src_rows, int64_t cols,
+                                     int64_t src_stride_row, const int64_t* row_index, int index_div,
+                                     const int64_t* offsets, const int64_t* pad_offsets, int num_experts,
+                                     void* dst, int64_t dst_stride, int64_t dst_cols, int apply_silu,
+                                     fmoe_stream_t stream) {
+    FMOE_REQUIRE(dtype == FMOE_BF16 || dtype == FMOE_F32, "fmoe_jagged_transpose: dtype must be bf16 or fp32");
+    FMOE_REQUIRE(src_rows >= 0 && cols >= 0 && dst_cols >= 0 && num_experts >= 1,
+                 "fmoe_jagged_transpose: negative extent or no experts");
+    FMOE_REQUIRE(index_div >= 1, "fmoe_jagged_transpose: index_div < 1");
+    if (cols == 0 || dst_cols == 0) return FMOE_OK;
+    FMOE_REQUIRE(src && offsets && pad_offsets && dst, "fmoe_jagged_transpose: NULL pointer");
+    FMOE_REQUIRE(src_stride_row >= cols && dst_stride >= dst_cols,
+                 "fmoe_jagged_transpose: a row stride is shorter than its row");
+    const int64_t gx = (dst_cols + 63) / 64, gy = (cols + 63) / 64;
+    FMOE_REQUIRE(gx < ((int64_t)1 << 31) && gy <= 65535, "fmoe_jagged_transpose: grid too large");
+    dim3 grid((unsigned)gx, (unsigned)gy);
+    if (dtype == FMOE_BF16)
+        jagged_transpose_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, src_rows, cols, src_stride_row, row_index, index_div, offsets, pad_offsets,
+            num_experts, (uint16_t*)dst, dst_stride, dst_cols, apply_silu);
+    else
+        jagged_transpose_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const float*)src, src_rows, cols, src_stride_row, row_index, index_div, offsets, pad_offsets,
+            num_experts, (float*)dst, dst_stride, dst_cols, apply_silu);
+    return check_launch("fmoe_jagged_transpose");
+}
+
+extern "C" int fmoe_segment_colsum(const void* src, int dtype, int64_t total_rows, int64_t cols,
+                                   int64_t src_stride_row, const int64_t* offsets, int num_experts, void* out,
+                                   fmoe_stream_t stream) {
+    FMOE_REQUIRE(dtype == FMOE_BF16 || dtype == FMOE_F32, "fmoe_segment_colsum: dtype must be bf16 or fp32");
+    FMOE_REQUIRE(total_rows >= 0 && cols >= 0 && num_experts >= 1 && num_experts <= 65535,
+                 "fmoe_segment_colsum: bad extents");
+    if (cols == 0) return FMOE_OK;
+    FMOE_REQUIRE((src || total_rows == 0) && offsets && out, "fmoe_segment_colsum: NULL pointer");
+    FMOE_REQUIRE(src_stride_row >= cols, "fmoe_segment_colsum: row stride shorter than the row");
+    dim3 grid((unsigned)((cols + 63) / 64), (unsigned)num_experts);
+    if (dtype == FMOE_BF16)
+        segment_colsum_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, total_rows, cols, src_stride_row, offsets, (uint16_t*)out);
+    else
+        segment_colsum_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const float*)src, total_rows, cols, src_stride_row, offsets, (float*)out);
+    return check_launch("fmoe_segment_colsum");
+}
+
+extern "C" int fmoe_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* du, int dtype,
+                               int64_t n, fmoe_stream_t stream) {
+    FMOE_REQUIRE(dtype == FMOE_BF16 || dtype == FMOE_F32, "fmoe_swiglu_bwd: dtype must be bf16 or fp32");
+    FMOE_REQUIRE(n >= 0, "fmoe_swiglu_bwd: n < 0");
+    if (n == 0) return FMOE_OK;
+    FMOE_REQUIRE(g && dh && dg && (!u || du), "fmoe_swiglu_bwd: NULL pointer");
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    FMOE_REQUIRE((n + 255) / 256 < ((int64_t)1 << 31), "fmoe_swiglu_bwd: too many elements");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FMOE_BF16) {
+        if (u) swiglu_bwd_kernel<uint16_t, true><<<blocks, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)u, (const uint16_t*)dh, (uint16_t*)dg, (uint16_t*)du, n);
+        else swiglu_bwd_kernel<uint16_t, false><<<blocks, 256, 0, s>>>((const uint16_t*)g, nullptr, (const uint16_t*)dh, (uint16_t*)dg, nullptr, n);
+    } else {
+        if (u) swiglu_bwd_kernel<float, true><<<blocks, 256, 0, s>>>((const float*)g, (const float*)u, (const float*)dh, (float*)dg, (float*)du, n);
+        else swiglu_bwd_kernel<float, false><<<blocks, 256, 0, s>>>((const float*)g, nullptr, (const float*)dh, (float*)dg, nullptr, n);
+    }
+    return check_launch("fmoe_swiglu_bwd");
+}
+
+extern "C" int fmoe_combine_bwd(const void* dy, const void* value, int value_dtype, int64_t T, int K, int64_t D,
+                                int64_t value_stride_row, const int64_t* token_index, const void* gates,
+                                int gates_dtype, int64_t gates_cols, int64_t gates_stride_row,
+                                int64_t gates_stride_col, const int64_t* gates_index, void* d_value,
+                                float* d_gates, fmoe_stream_t stream) {
+    FMOE_REQUIRE(value_dtype == FMOE_BF16 || value_dtype == FMOE_F32, "fmoe_combine_bwd: value must be bf16 or fp32");
+    FMOE_REQUIRE(T >= 0 && K >= 1 && D >= 1, "fmoe_combine_bwd: need T >= 0, K >= 1, D >= 1");
+    if (T == 0) return FMOE_OK;
+    FMOE_REQUIRE(dy && token_index && d_value, "fmoe_combine_bwd: NULL pointer");
+    FMOE_REQUIRE(!d_gates || (value && value_stride_row >= D), "fmoe_combine_bwd: d_gates needs value rows");
+    if (gates) {
+        FMOE_REQUIRE(gates_dtype == FMOE_BF16 || gates_dtype == FMOE_F32, "fmoe_combine_bwd: gates must be bf16 or fp32");
+        FMOE_REQUIRE(gates_cols >= 1, "fmoe_combine_bwd: gates_cols < 1");
+    }
+    const int64_t R = T * (int64_t)K;
+    FMOE_REQUIRE((R + 3) / 4 < ((int64_t)1 << 31), "fmoe_combine_bwd: too many rows");
+    GateArgs ga{gates, gates_cols, gates_stride_row, gates_stride_col, gates_index, R};
+    const unsigned blocks = (unsigned)((R + 3) / 4);
+    hipStream_t s = (hipStream_t)stream;
+    const bool gb = gates && gates_dtype == FMOE_BF16;
+    if (value_dtype == FMOE_BF16) {
+        if (gb) combine_bwd_kernel<uint16_t, uint16_t><<<blocks, 256, 0, s>>>((const uint16_t*)dy, (const uint16_t*)value, T, R, D, value_stride_row, token_index, ga, (uint16_t*)d_value, d_gates);
+        else combine_bwd_kernel<uint16_t, float><<<blocks, 256, 0, s>>>((const uint16_t*)dy, (const uint16_t*)value, T, R, D, value_stride_row, token_index, ga, (uint16_t*)d_value, d_gates);
+    } else {
+        if (gb) combine_bwd_kernel<float, uint16_t><<<blocks, 256, 0, s>>>((const float*)dy, (const float*)value, T, R, D, value_stride_row, token_index, ga, (float*)d_value, d_gates);
+        else combine_bwd_kernel<float, float><<<blocks, 256, 0, s>>>((const float*)dy, (const float*)value, T, R, D, value_stride_row, token_index, ga, (float*)d_value, d_gates);
+    }
+    return check_launch("fmoe_combine_bwd");
+}

@@ -90,6 +90,7 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     p.n_tiles = 0;
     // 16-byte stores: 8 bf16 (4 fp32) output columns at a time
     const int vec_cols = f32 ? 4 : 8;
+    p.k_window = d->k_window;
     p.vec_store = (d->n % vec_cols == 0) && (d->out_stride_row % vec_cols == 0) && aligned16(d->out);
 
     const int esize = fp8 ? 1 : (f32 ? 4 : 2);
@@ -107,7 +108,7 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     const int64_t span32 = ((int64_t)1 << 32) - 4096;
     const bool near = d->a_rows * d->a_stride_row * esize + (int64_t)d->k * esize < span32 &&
                       (int64_t)d->n * d->b_stride_n * esize + (int64_t)d->k * esize < span32;
-    const bool ring = fast && big && !f32 && !d->a_silu && (d->k % slice) == 0 && d->k / slice >= 3 &&
+    const bool ring = fast && big && !f32 && !d->a_silu && !d->k_window && (d->k % slice) == 0 && d->k / slice >= 3 &&
                       p.vec_store && d->num_experts <= 1024 && d->total_rows < ((int64_t)1 << 31) * 128 && near;
     const int sel = !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
     if (fp8) return run_gemm_fp8(p, d->epilogue, sel, stream);

@@ -64,6 +64,7 @@ struct GemmParams {
     int64_t out_stride;
     int n_tiles;
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
+    const int64_t* k_window;            // [E+1] per-expert contraction range, or null
 };
 
 constexpr int kDtBf16 = 0, kDtE4m3 = 1, kDtF32 = 2;
@@ -349,8 +350,17 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
     }
     if (rows_valid <= 0) return;   // unreachable for consistent offsets
 
+    // per-expert contraction window (weight gradients): both operands start k_begin elements in
+    int Kdim = p.K;
+    int64_t k_begin = 0;
+    if (p.k_window) {
+        k_begin = p.k_window[expert];
+        const int64_t span = p.k_window[expert + 1] - k_begin;
+        Kdim = (int)(span < 0 ? 0 : (span < p.K ? span : p.K));
+    }
+
     // --------------------------------------------------------------- loaders
-    const uint8_t* a_base = p.a + (int64_t)expert * p.a_stride_e * ESIZE;
+    const uint8_t* a_base = p.a + ((int64_t)expert * p.a_stride_e + k_begin) * ESIZE;
     const int64_t a_row_bytes = p.a_stride_row * ESIZE;
     const int n0 = nt * BN_OUT;
 
@@ -393,27 +403,27 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
         else { const int q = tid + i * NT; row = q % BN; chunk = q / BN; }
         const uint8_t* base;
         const int n = w_row_of(row, base);
-        wptr[i] = base + ((int64_t)expert * p.b_se + (int64_t)n * p.b_sn) * ESIZE;
+        wptr[i] = base + ((int64_t)expert * p.b_se + (int64_t)n * p.b_sn + k_begin * p.b_sk) * ESIZE;
         woff[i] = BM * 128 + lds_off(row, chunk);
         wchunk[i] = chunk;
     }
 
     u32x4 xr[XP], wr[WP];
     auto load_global = [&](int kt) {
-        const bool whole = (kt + 1) * BK <= p.K;      // uniform: no per-lane predicate inside K
+        const bool whole = (kt + 1) * BK <= Kdim;      // uniform: no per-lane predicate inside K
 #pragma unroll
         for (int i = 0; i < XP; ++i) {
             const int k = kt * BK + xchunk[i] * CHUNK_ELEMS;
             if (FAST) {
                 if (whole) xr[i] = *reinterpret_cast<const u32x4*>(xptr[i] + (int64_t)k * ESIZE);
-                else xr[i] = k < p.K ? *reinterpret_cast<const u32x4*>(xptr[i] + (int64_t)k * ESIZE)
+                else xr[i] = k < Kdim ? *reinterpret_cast<const u32x4*>(xptr[i] + (int64_t)k * ESIZE)
                                      : u32x4{0, 0, 0, 0};
             } else {
                 uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
                 for (int j = 0; j < CHUNK_ELEMS; ++j) {
                     uint32_t v = 0;
-                    if (k + j < p.K)
+                    if (k + j < Kdim)
                         v = FP8 ? (uint32_t)xptr[i][k + j]
                             : F32 ? reinterpret_cast<const uint32_t*>(xptr[i])[k + j]
                                   : (uint32_t) reinterpret_cast<const uint16_t*>(xptr[i])[k + j];
@@ -428,14 +438,14 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
             const int k = kt * BK + wchunk[i] * CHUNK_ELEMS;
             if (FAST) {
                 if (whole) wr[i] = *reinterpret_cast<const u32x4*>(wptr[i] + (int64_t)k * ESIZE);
-                else wr[i] = k < p.K ? *reinterpret_cast<const u32x4*>(wptr[i] + (int64_t)k * ESIZE)
+                else wr[i] = k < Kdim ? *reinterpret_cast<const u32x4*>(wptr[i] + (int64_t)k * ESIZE)
                                      : u32x4{0, 0, 0, 0};
             } else {
                 uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
                 for (int j = 0; j < CHUNK_ELEMS; ++j) {
                     uint32_t v = 0;
-                    if (k + j < p.K) {
+                    if (k + j < Kdim) {
                         const int64_t off = (int64_t)(k + j) * p.b_sk;
                         v = FP8 ? (uint32_t)wptr[i][off]
                             : F32 ? reinterpret_cast<const uint32_t*>(wptr[i])[off]
@@ -477,7 +487,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
     for (int fm = 0; fm < FM; ++fm) xfrag_row[fm] = wm * TM + fm * 32 + (lane & 31);
     const int khalf = lane >> 5;
 
-    const int KT = (p.K + BK - 1) / BK;
+    const int KT = (Kdim + BK - 1) / BK;
     load_global(0);
     store_lds(0);
     __syncthreads();

@@ -19,7 +19,8 @@ EPI_NONE, EPI_SILU, EPI_SWIGLU = 0, 1, 2
 EXPORTED_SYMBOLS = (
     "fmoe_version", "fmoe_last_error", "fmoe_route_workspace_bytes", "fmoe_route_topk",
     "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_combine",
-    "fmoe_silu_mul", "fmoe_transpose_last2",
+    "fmoe_silu_mul", "fmoe_transpose_last2", "fmoe_jagged_transpose", "fmoe_segment_colsum",
+    "fmoe_swiglu_bwd", "fmoe_combine_bwd",
 )
 
 
@@ -37,6 +38,7 @@ class GemmDesc(ctypes.Structure):
         ("bias", c_void_p), ("bias2", c_void_p), ("bias_stride_e", c_int64),
         ("epilogue", c_int32), ("out_dtype", c_int32),
         ("out", c_void_p), ("out_stride_row", c_int64),
+        ("k_window", c_void_p),
     ]
 
 
@@ -78,6 +80,18 @@ def load() -> ctypes.CDLL:
     lib.fmoe_transpose_last2.restype = c_int
     lib.fmoe_transpose_last2.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
                                          c_void_p]
+    lib.fmoe_jagged_transpose.restype = c_int
+    lib.fmoe_jagged_transpose.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
+                                          c_void_p, c_int, c_void_p, c_int64, c_int64, c_int, c_void_p]
+    lib.fmoe_segment_colsum.restype = c_int
+    lib.fmoe_segment_colsum.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
+                                        c_void_p]
+    lib.fmoe_swiglu_bwd.restype = c_int
+    lib.fmoe_swiglu_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_void_p]
+    lib.fmoe_combine_bwd.restype = c_int
+    lib.fmoe_combine_bwd.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_int64, c_void_p,
+                                     c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+                                     c_void_p]
     _lib = lib
     return lib
 

@@ -1,0 +1,178 @@
+"""Backward of the MoE operators on the HIP back-end (torch.autograd.Function wrappers).
+
+What the reference's Triton autograd functions compute
+(/root/reference/kernels/triton/triton_moe.py:606-804 index_select_jagged_bmm backward,
+:62-141 fused SwiGLU backward, :922-983 merge backward, :3790-4027 silu_jagged_bmm_combine
+backward), built from the library's kernels:
+
+* input gradient  = grouped GEMM of the output gradient with the transposed weight, then the
+  deterministic gather-form sum of the K routed rows of every token (fmoe_combine);
+* weight gradient = grouped GEMM with a per-expert contraction window over the rows of the
+  expert (fmoe_grouped_gemm + k_window) on operands that fmoe_jagged_transpose laid out
+  K-contiguous and zero padded;
+* bias gradient   = fmoe_segment_colsum; activation and merge backward = fmoe_swiglu_bwd,
+  fmoe_combine_bwd.
+
+torch is used for index bookkeeping on [E]- and [T, K]-sized integer tensors only.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import ops
+from ._lib import EPI_NONE, EPI_SWIGLU
+
+
+def _pad_layout(offsets: torch.Tensor, total_rows: int) -> Tuple[torch.Tensor, int]:
+    """Per-expert row counts rounded up to 8 -> (padded prefix [E+1], host-side bound of its end)."""
+    lengths = (offsets[1:] - offsets[:-1]).clamp_min(0)
+    padded = (lengths + 7) // 8 * 8
+    pad_offsets = torch.zeros_like(offsets)
+    pad_offsets[1:] = torch.cumsum(padded, 0)
+    E = offsets.numel() - 1
+    bound = (total_rows + 8 * E + 63) // 64 * 64
+    return pad_offsets, bound
+
+
+def _reverse_from_index(index: torch.Tensor) -> torch.Tensor:
+    """index [T, K] (sorted position -> flat token*K+slot) -> [T, K] sorted positions of each
+    token's rows, ascending (the order a sequential index_add meets them in)."""
+    T, K = index.shape
+    flat = index.reshape(-1)
+    inv = torch.empty_like(flat)
+    inv[flat] = torch.arange(flat.numel(), device=flat.device, dtype=flat.dtype)
+    return inv.view(T, K).sort(dim=1).values
+
+
+def weight_grad(a_src: torch.Tensor, dout: torch.Tensor, offsets: torch.Tensor, *,
+                row_index: Optional[torch.Tensor] = None, index_div: int = 1,
+                apply_silu: bool = False) -> torch.Tensor:
+    """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a(r)[k], a(r) = the (gathered,
+    optionally SiLU-ed) input row of routed row r.  Returns [E, N, K] contiguous."""
+    R, N = dout.shape
+    Kin = a_src.shape[1]
+    E = offsets.numel() - 1
+    pad_offsets, bound = _pad_layout(offsets, R)
+    dout_t = ops.jagged_transpose(dout, offsets, pad_offsets, bound)                       # [N, bound]
+    a_t = ops.jagged_transpose(a_src, offsets, pad_offsets, bound, row_index, index_div, apply_silu)  # [Kin, bound]
+    dev = dout.device
+    seg = torch.arange(E + 1, device=dev, dtype=torch.int64) * N
+    rows = torch.arange(E * N, device=dev, dtype=torch.int64) % N
+    b = a_t.t().unsqueeze(0).expand(E, bound, Kin)                                          # B[e, k, n'] = a_t[n', k]
+    dw = ops.grouped_gemm(seg, dout_t, b, total_rows=E * N, row_index=rows, index_div=1, epilogue=EPI_NONE,
+                          k_window=pad_offsets)
+    return dw.view(E, N, Kin)
+
+
+def _input_grad(drow_list, weights, offsets, reverse_index) -> torch.Tensor:
+    """sum over branches and over the K rows of a token of drow @ W^T -> [T, K_in]."""
+    R = drow_list[0].shape[0]
+    parts = [ops.grouped_gemm(offsets, d, w.permute(0, 2, 1), total_rows=R) for d, w in zip(drow_list, weights)]
+    if len(parts) == 1:
+        return ops.combine(parts[0], reverse_index)
+    value = torch.cat(parts, dim=0)
+    rev = torch.cat([reverse_index + i * R for i in range(len(parts))], dim=1)
+    return ops.combine(value, rev)
+
+
+class IndexSelectJaggedBmm(torch.autograd.Function):
+    """index_select_jagged_bmm and index_select_jagged_bmm_swiglu (weight_p is None or not)."""
+
+    @staticmethod
+    def forward(ctx, offsets, index, jagged, weight, bias, weight_p, bias_p):
+        swiglu = weight_p is not None
+        out = ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
+                               index_div=index.shape[-1], bias=bias, b2=weight_p, bias2=bias_p,
+                               epilogue=EPI_SWIGLU if swiglu else EPI_NONE)
+        ctx.save_for_backward(offsets, index, jagged, weight, bias, weight_p, bias_p)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        offsets, index, jagged, weight, bias, weight_p, bias_p = ctx.saved_tensors
+        K = index.shape[-1]
+        R = index.numel()
+        dout = dout.contiguous()
+        swiglu = weight_p is not None
+        if swiglu:   # the pre-activations are recomputed, not kept from the forward
+            gemm = lambda w, b: ops.grouped_gemm(offsets, jagged, w, total_rows=R, row_index=index,
+                                                 index_div=K, bias=b)
+            g, u = gemm(weight, bias), gemm(weight_p, bias_p)
+            dg, du = ops.swiglu_bwd(g, u, dout)
+            drows, weights = [dg, du], [weight, weight_p]
+        else:
+            drows, weights = [dout], [weight]
+        need = ctx.needs_input_grad
+        d_jagged = d_w = d_b = d_wp = d_bp = None
+        if need[2]:
+            d_jagged = _input_grad(drows, weights, offsets, _reverse_from_index(index)).view_as(jagged)
+        flat_index = index.reshape(-1)
+        if need[3]:
+            d_w = weight_grad(jagged, drows[0], offsets, row_index=flat_index, index_div=K).permute(0, 2, 1)
+        if bias is not None and need[4]:
+            d_b = ops.segment_colsum(drows[0], offsets)
+        if swiglu and need[5]:
+            d_wp = weight_grad(jagged, drows[1], offsets, row_index=flat_index, index_div=K).permute(0, 2, 1)
+        if swiglu and bias_p is not None and need[6]:
+            d_bp = ops.segment_colsum(drows[1], offsets)
+        return None, None, d_jagged, d_w, d_b, d_wp, d_bp
+
+
+class MulMergeKAdd(torch.autograd.Function):
+    """mul_merge_k_add: weighted deterministic merge."""
+
+    @staticmethod
+    def forward(ctx, index, reverse_index, value, weight, weight_index):
+        out = ops.combine(value, reverse_index, weight, weight_index)
+        ctx.save_for_backward(index, value, weight, weight_index)
+        ctx.K = reverse_index.shape[1]
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        index, value, weight, weight_index = ctx.saved_tensors
+        need_w = weight is not None and ctx.needs_input_grad[3]
+        dy = dy.to(value.dtype)
+        d_value, d_gate = ops.combine_bwd(dy, value, index, ctx.K, weight, weight_index, need_gate_grad=need_w)
+        d_weight = d_gate.view(weight.shape).to(weight.dtype) if need_w else None
+        return None, None, d_value if ctx.needs_input_grad[2] else None, d_weight, None
+
+
+class SiluJaggedBmmCombine(torch.autograd.Function):
+    """silu_jagged_bmm_combine: (SiLU,) grouped GEMM + bias, weighted merge."""
+
+    @staticmethod
+    def forward(ctx, offsets, jagged, weight, bias, index, reverse_index, gating_scores, gates_index, has_silu):
+        bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
+                                   epilogue=EPI_NONE, a_silu=has_silu)
+        out = ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
+        ctx.save_for_backward(offsets, jagged, weight, bias, index, gating_scores, gates_index, bmm_out)
+        ctx.has_silu = has_silu
+        ctx.K = reverse_index.shape[1]
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        offsets, jagged, weight, bias, index, gating_scores, gates_index, bmm_out = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        need_g = gating_scores is not None and need[6]
+        dy = dy.to(bmm_out.dtype)
+        d_bmm, d_gate = ops.combine_bwd(dy, bmm_out, index, ctx.K, gating_scores, gates_index,
+                                        need_gate_grad=need_g)
+        d_jagged = d_w = d_b = d_g = None
+        if need[1]:
+            d_h = ops.grouped_gemm(offsets, d_bmm, weight.permute(0, 2, 1), total_rows=d_bmm.shape[0])
+            d_jagged = ops.swiglu_bwd(jagged, None, d_h)[0] if ctx.has_silu else d_h
+        if need[2]:
+            d_w = weight_grad(jagged, d_bmm, offsets, apply_silu=ctx.has_silu).permute(0, 2, 1)
+        if bias is not None and need[3]:
+            d_b = ops.segment_colsum(d_bmm, offsets)
+        if need_g:
+            d_g = d_gate.view(gating_scores.shape).to(gating_scores.dtype)
+        return None, d_jagged, d_w, d_b, None, None, d_g, None, None
+
+
+def needs_grad(*tensors: Optional[torch.Tensor]) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)

@@ -180,7 +180,8 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  bias: Optional[torch.Tensor] = None, b2: Optional[torch.Tensor] = None,
                  bias2: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE, a_silu: bool = False,
                  a_scale: Optional[torch.Tensor] = None, b_scale: Optional[torch.Tensor] = None,
-                 b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0) -> torch.Tensor:
+                 b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0,
+                 k_window: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
     strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
     [total_rows, N] in bf16 (fp32 for fp32 operands)."""
@@ -206,7 +207,11 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     a = _rows_contiguous(a)
     # N-contiguous weights of a useful size: one transposing copy buys the streaming kernel
     # (the element-load kernel that reads them in place is correct but an order of magnitude slower)
-    if b.stride(2) == 1 and b.stride(1) != 1 and K % 16 == 0 and N % 8 == 0 and total_rows * N >= (1 << 22):
+    if k_window is not None:
+        k_window = _i64("k_window", k_window)
+        if k_window.numel() != E + 1:
+            raise ValueError(f"grouped_gemm: k_window must have E+1={E + 1} entries")
+    elif b.stride(2) == 1 and b.stride(1) != 1 and K % 16 == 0 and N % 8 == 0 and total_rows * N >= (1 << 22):
         b = to_k_contiguous(b)
         if b2 is not None:
             b2 = to_k_contiguous(b2)
@@ -264,6 +269,7 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.out_dtype = _DTYPE_CODE[out_dtype]
     d.out = out.data_ptr()
     d.out_stride_row = out.stride(0)
+    d.k_window = _ptr(k_window)
     rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
     _lib.check(rc, "fmoe_grouped_gemm")
     return out
@@ -319,3 +325,99 @@ def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
                                    _stream(a))
     _lib.check(rc, "fmoe_silu_mul")
     return out
+
+
+# ----------------------------------------------------------------- backward
+def jagged_transpose(src: torch.Tensor, offsets: torch.Tensor, pad_offsets: torch.Tensor, padded_cols: int,
+                     row_index: Optional[torch.Tensor] = None, index_div: int = 1,
+                     apply_silu: bool = False) -> torch.Tensor:
+    """[rows, C] jagged rows (optionally gathered) -> [C, padded_cols] transposed and zero padded per
+    expert, see fmoe_jagged_transpose."""
+    dev = _need_cuda("jagged_transpose", src, offsets, pad_offsets, row_index)
+    if src.ndim != 2 or src.dtype not in _DTYPE_CODE:
+        raise ValueError("jagged_transpose: src must be a 2-D bf16 or fp32 tensor")
+    src = _rows_contiguous(src)
+    offsets, pad_offsets = _i64("offsets", offsets), _i64("pad_offsets", pad_offsets)
+    if row_index is not None:
+        row_index = _i64("row_index", row_index).view(-1)
+    E = offsets.numel() - 1
+    C = src.shape[1]
+    dst = torch.empty((C, padded_cols), dtype=src.dtype, device=dev)
+    rc = _lib.load().fmoe_jagged_transpose(
+        src.data_ptr(), _DTYPE_CODE[src.dtype], src.shape[0], C, src.stride(0), _ptr(row_index), index_div,
+        offsets.data_ptr(), pad_offsets.data_ptr(), E, dst.data_ptr(), dst.stride(0), padded_cols,
+        int(apply_silu), _stream(src))
+    _lib.check(rc, "fmoe_jagged_transpose")
+    return dst
+
+
+def segment_colsum(src: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+    """Per-expert column sums [E, C] of jagged rows [R, C], see fmoe_segment_colsum."""
+    dev = _need_cuda("segment_colsum", src, offsets)
+    if src.ndim != 2 or src.dtype not in _DTYPE_CODE:
+        raise ValueError("segment_colsum: src must be a 2-D bf16 or fp32 tensor")
+    src = _rows_contiguous(src)
+    offsets = _i64("offsets", offsets)
+    E = offsets.numel() - 1
+    out = torch.empty((E, src.shape[1]), dtype=src.dtype, device=dev)
+    rc = _lib.load().fmoe_segment_colsum(src.data_ptr(), _DTYPE_CODE[src.dtype], src.shape[0], src.shape[1],
+                                         src.stride(0), offsets.data_ptr(), E, out.data_ptr(), _stream(src))
+    _lib.check(rc, "fmoe_segment_colsum")
+    return out
+
+
+def swiglu_bwd(g: torch.Tensor, u: Optional[torch.Tensor], dh: torch.Tensor):
+    """Backward of ``silu(g) * u`` (or of ``silu(g)`` when u is None): returns (dg, du)."""
+    _need_cuda("swiglu_bwd", g, u, dh)
+    if g.dtype not in _DTYPE_CODE or dh.dtype != g.dtype or dh.shape != g.shape or (
+            u is not None and (u.dtype != g.dtype or u.shape != g.shape)):
+        raise ValueError("swiglu_bwd: bf16 (or fp32) tensors of one shape expected")
+    g, dh = g.contiguous(), dh.contiguous()
+    u = None if u is None else u.contiguous()
+    dg = torch.empty_like(g)
+    du = None if u is None else torch.empty_like(g)
+    rc = _lib.load().fmoe_swiglu_bwd(g.data_ptr(), _ptr(u), dh.data_ptr(), dg.data_ptr(), _ptr(du),
+                                     _DTYPE_CODE[g.dtype], g.numel(), _stream(g))
+    _lib.check(rc, "fmoe_swiglu_bwd")
+    return dg, du
+
+
+def combine_bwd(dy: torch.Tensor, value: Optional[torch.Tensor], token_index: torch.Tensor, K: int,
+                gates: Optional[torch.Tensor] = None, gates_index: Optional[torch.Tensor] = None,
+                need_gate_grad: bool = False):
+    """Backward of ``combine``: (d_value [T*K, D], d_gates fp32 [T*K] in the gates' flat layout or None)."""
+    dev = _need_cuda("combine_bwd", dy, value, token_index, gates, gates_index)
+    if dy.ndim != 2 or dy.dtype not in _DTYPE_CODE:
+        raise ValueError("combine_bwd: dy must be a 2-D bf16 or fp32 tensor")
+    dy = dy.contiguous()
+    T, D = dy.shape
+    R = T * K
+    token_index = _i64("token_index", token_index).view(-1)
+    if token_index.numel() != R:
+        raise ValueError("combine_bwd: token_index must have T*K entries")
+    g_code, g_cols, g_sr, g_sc = FMOE_F32, 1, 1, 1
+    if gates is not None:
+        if gates.dtype not in _DTYPE_CODE or gates.numel() != R:
+            raise ValueError("combine_bwd: gates must be bf16 / fp32 with T*K entries")
+        if gates.ndim != 2:
+            gates = gates.contiguous().view(-1, 1)
+        g_code, g_cols, g_sr, g_sc = _DTYPE_CODE[gates.dtype], gates.shape[1], gates.stride(0), gates.stride(1)
+        if gates_index is not None:
+            gates_index = _i64("gates_index", gates_index).view(-1)
+    else:
+        gates_index = None
+    d_gates = None
+    v_stride = D
+    if need_gate_grad:
+        if value is None or value.dtype != dy.dtype or tuple(value.shape) != (R, D):
+            raise ValueError("combine_bwd: the gate gradient needs value [T*K, D] in dy's dtype")
+        value = _rows_contiguous(value)
+        v_stride = value.stride(0)
+        d_gates = torch.zeros((R,), dtype=torch.float32, device=dev)
+    d_value = torch.empty((R, D), dtype=dy.dtype, device=dev)
+    rc = _lib.load().fmoe_combine_bwd(
+        dy.data_ptr(), _ptr(value) if need_gate_grad else None, _DTYPE_CODE[dy.dtype], T, K, D, v_stride,
+        token_index.data_ptr(), _ptr(gates), g_code, g_cols, g_sr, g_sc, _ptr(gates_index), d_value.data_ptr(),
+        _ptr(d_gates), _stream(dy))
+    _lib.check(rc, "fmoe_combine_bwd")
+    return d_value, d_gates

@@ -6,7 +6,10 @@ of /root/reference/kernels/moe.py:39-292.  Differences, all on purpose:
 * ``kernel`` defaults to ``KernelType.HIP`` (the reference defaults to its
   PyTorch path, which this package does not contain); ``KernelType.TRITON`` is
   accepted and runs the same HIP kernels; any other value raises.
-* forward only: inputs that require grad raise unless grad mode is off.
+* backward is implemented for index_select_jagged_bmm, index_select_jagged_bmm_swiglu,
+  mul_merge_k_add and silu_jagged_bmm_combine (kernels/hip/autograd.py); the 3D and
+  two-input gating variants and the fp8 operators are forward only and raise when an
+  input requires grad under grad mode.
 * ``max_seq_len`` is accepted and ignored: tile scheduling reads ``offsets`` on
   the device, so no host synchronisation is needed to obtain it.
 * operands must be bf16 or fp32 CUDA tensors (fp32 runs true-fp32 MFMA, no tf32).
@@ -18,6 +21,7 @@ from typing import Optional
 
 import torch
 
+from .hip import autograd as _ag
 from .hip import ops
 from .hip._lib import EPI_NONE, EPI_SWIGLU
 from .utils import KernelType, require_hip_kernel
@@ -62,7 +66,8 @@ def index_select_jagged_bmm(
     """kernels/moe.py:39-68.  ``out[off_e:off_e+1] = jagged[index[...] // A] @ weight[e] + bias[e]``."""
     require_hip_kernel(kernel, "index_select_jagged_bmm")
     _check_gather_args("index_select_jagged_bmm", index, jagged, weight)
-    ops._forward_only("index_select_jagged_bmm", jagged, weight, bias)
+    if _ag.needs_grad(jagged, weight, bias):
+        return _ag.IndexSelectJaggedBmm.apply(offsets, index, jagged, weight, bias, None, None)
     return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                             index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
 
@@ -88,7 +93,8 @@ def mul_merge_k_add(
         assert weight_index is not None
         assert weight.numel() == weight_index.numel() == value.shape[0], (
             f"{weight.shape=}, {weight_index.shape=}, {value.shape=}")
-    ops._forward_only("mul_merge_k_add", value, weight)
+    if _ag.needs_grad(value, weight):
+        return _ag.MulMergeKAdd.apply(index, reverse_index, value, weight, weight_index)
     return ops.combine(value, reverse_index, weight, weight_index)
 
 
@@ -127,10 +133,11 @@ def index_select_jagged_bmm_swiglu(
     require_hip_kernel(kernel, "index_select_jagged_bmm_swiglu")
     _check_gather_args("index_select_jagged_bmm_swiglu", index, jagged, weight)
     assert weight.shape == weight_p.shape
-    ops._forward_only("index_select_jagged_bmm_swiglu", jagged, weight, bias, weight_p, bias_p)
     if weight_p.stride() != weight.stride():
         weight_p = weight_p.contiguous()
         weight = weight.contiguous()
+    if _ag.needs_grad(jagged, weight, bias, weight_p, bias_p):
+        return _ag.IndexSelectJaggedBmm.apply(offsets, index, jagged, weight, bias, weight_p, bias_p)
     return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                             index_div=index.shape[-1], bias=bias, b2=weight_p, bias2=bias_p,
                             epilogue=EPI_SWIGLU)
@@ -187,7 +194,9 @@ def silu_jagged_bmm_combine(
     L, K = reverse_index.shape
     assert index.ndim == 1 and reverse_index.ndim == 2
     assert N == L * K and N == jagged.shape[0], f"{N=}, {L=}, {K=}, {jagged.shape=}"
-    ops._forward_only("silu_jagged_bmm_combine", jagged, weight, bias, gating_scores)
+    if _ag.needs_grad(jagged, weight, bias, gating_scores):
+        return _ag.SiluJaggedBmmCombine.apply(offsets, jagged, weight, bias, index, reverse_index,
+                                              gating_scores, gates_index, has_silu)
     bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=N, bias=bias, epilogue=EPI_NONE,
                                a_silu=has_silu)
     return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)

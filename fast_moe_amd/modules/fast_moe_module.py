@@ -82,11 +82,35 @@ class FastMoELayer(nn.Module):
         qo, so = cached_quantize_expert_weights(self._experts_w.permute(0, 2, 1))
         return {"hidden_w": qh, "hidden_scale": sh, "out_w": qo, "out_scale": so}
 
+    def _forward_with_grad(self, x: torch.Tensor, k: int) -> torch.Tensor:
+        """The two-operator form of fast_moe_module.py:146-186 on the differentiable HIP operators
+        (same values as ``forward``: the fused SiLU epilogue rounds where this form rounds).  The
+        routing integers come from the library; the K gate values are re-derived from the gate
+        probabilities with torch ops so that the gate network receives its gradient
+        (fast_moe_module.py:93-105: mask, then L1 normalisation)."""
+        from ..kernels import moe
+        if x.dtype not in (torch.bfloat16, torch.float32):
+            raise NotImplementedError(f"FastMoELayer: the HIP kernels take bf16 or fp32 activations, got {x.dtype}")
+        original_shape = x.shape
+        scores = self.gate(x).reshape(-1, self.num_experts)
+        r = ops.route_topk(scores.detach(), k, renorm=True)
+        picked = scores.gather(1, r["topk_idx"])
+        gates = picked / picked.sum(dim=1, keepdim=True).clamp_min(1e-12)
+        x_flat = x.reshape(-1, self.input_dim)
+        T = x_flat.shape[0]
+        hidden = moe.index_select_jagged_bmm(
+            0, r["offsets"], r["gate_index"].view(T, k), x_flat,
+            self._experts_hidden_w.permute(0, 2, 1).to(x.dtype), self._experts_hidden_bias.to(x.dtype))
+        y = moe.silu_jagged_bmm_combine(
+            0, r["offsets"], hidden, self._experts_w.permute(0, 2, 1).to(x.dtype),
+            self._experts_bias.to(x.dtype), r["token_index"], r["reverse_index"], gates, r["gate_index"],
+            has_silu=True)
+        return y.view(original_shape[0], original_shape[1], self.output_dim)
+
     def forward(self, x: torch.Tensor, num_experts_per_tok: int) -> torch.Tensor:
         require_hip_kernel(self.kernel, "FastMoELayer.forward")
         if torch.is_grad_enabled() and (x.requires_grad or any(p.requires_grad for p in self.parameters())):
-            raise RuntimeError("FastMoELayer: the HIP back-end is forward-only; call it under "
-                               "torch.no_grad() / torch.inference_mode()")
+            return self._forward_with_grad(x, num_experts_per_tok)
         if x.dtype not in (torch.bfloat16, torch.float32):
             raise NotImplementedError(f"FastMoELayer: the HIP kernels take bf16 or fp32 activations, got {x.dtype}")
         original_shape = x.shape

@@ -148,6 +148,11 @@ int fmoe_quant_rows_e4m3(const void* a, int a_dtype, int64_t batch, int64_t rows
  * + n*b_stride_n], so both [E,K,N]-contiguous weights and [E,K,N] views of
  * [E,N,K] storage are consumed in place.  No host synchronisation: tile
  * scheduling reads `offsets` on the device; max_seq_len is not needed.
+ *
+ * With k_window the contraction range differs per expert: this is the weight
+ * gradient of the operators above, dW[e] = A_e^T x dOut_e reduced over the rows of
+ * expert e (kernels/triton/triton_moe.py:1793-1976, 4030-4108), computed on the
+ * transposed, zero-padded operands fmoe_jagged_transpose writes.
  */
 typedef struct fmoe_gemm_desc {
     int32_t num_experts;    /* E                                                  */
@@ -180,6 +185,9 @@ typedef struct fmoe_gemm_desc {
     int32_t out_dtype;      /* FMOE_BF16; FMOE_F32 iff a_dtype is FMOE_F32        */
     void* out;              /* [total_rows, n]                                    */
     int64_t out_stride_row;
+    const int64_t* k_window; /* NULL, or [E+1]: expert e contracts over the k range
+                                [k_window[e], k_window[e+1]) of A and B (then `k` is
+                                only an upper bound); values multiples of 8          */
 } fmoe_gemm_desc;
 
 int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);
@@ -226,6 +234,59 @@ int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
  */
 int fmoe_transpose_last2(const void* src, void* dst, int elem_size, int64_t batch, int64_t rows,
                          int64_t cols, int64_t src_stride_b, int64_t src_stride_r, fmoe_stream_t stream);
+
+/* ----------------------------------------------------------------- backward */
+
+/*
+ * Transposed, zero-padded copy of jagged rows, the operand layout of the weight-gradient GEMM:
+ *   for e in [0, E), j in [0, len_e):  dst[c, pad_offsets[e] + j] = src[src_row(offsets[e] + j), c]
+ *   dst[c, p] = 0 for the padding columns p in [pad_offsets[e] + len_e, pad_offsets[e+1])
+ * with len_e = offsets[e+1] - offsets[e] and src_row(r) = row_index ? row_index[r] / index_div : r;
+ * apply_silu != 0 stores silu(src) (rounded to dtype) instead, for the operator whose GEMM input
+ * is silu(jagged) (kernels/pytorch/moe.py:255-275).
+ * The reference's jagged x jagged kernels read both operands strided
+ * (kernels/triton/triton_moe.py:1793-1976); here the reduction index is made contiguous once.
+ *   src          [src_rows, cols], FMOE_BF16 or FMOE_F32, cols contiguous
+ *   pad_offsets  [E+1], pad_offsets[e+1] - pad_offsets[e] >= len_e
+ *   dst          [cols, dst_stride], columns [0, dst_cols) are written (dst_cols >= pad_offsets[E],
+ *                a host-side bound; columns past pad_offsets[E] are zeroed)
+ */
+int fmoe_jagged_transpose(const void* src, int dtype, int64_t src_rows, int64_t cols,
+                          int64_t src_stride_row, const int64_t* row_index, int index_div,
+                          const int64_t* offsets, const int64_t* pad_offsets, int num_experts,
+                          void* dst, int64_t dst_stride, int64_t dst_cols, int apply_silu,
+                          fmoe_stream_t stream);
+
+/*
+ * out[e, c] = sum over r in [offsets[e], offsets[e+1]) of src[r, c], fp32 accumulation in a
+ * fixed order: the bias gradient of the grouped GEMMs (torch autograd's sum over the rows of
+ * each F.linear call in kernels/pytorch/moe.py:75-82).  src / out FMOE_BF16 or FMOE_F32.
+ */
+int fmoe_segment_colsum(const void* src, int dtype, int64_t total_rows, int64_t cols,
+                        int64_t src_stride_row, const int64_t* offsets, int num_experts, void* out,
+                        fmoe_stream_t stream);
+
+/*
+ * Element-wise backward of h = silu(g) * u (the SwiGLU epilogue; kernels/triton/triton_moe.py:62-141):
+ *   du = dh * silu(g),   dg = (dh * u) * sigmoid(g) * (1 + g * (1 - sigmoid(g)))
+ * rounded where torch autograd rounds (silu(g), dh * u and both results in `dtype`).
+ * u == NULL: plain SiLU backward, dg = dh * sigmoid(g) * (1 + g * (1 - sigmoid(g))), du unused.
+ */
+int fmoe_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* du, int dtype,
+                    int64_t n, fmoe_stream_t stream);
+
+/*
+ * Backward of fmoe_combine (kernels/triton/triton_moe.py:922-983): for every routed row r with
+ * t = token_index[r] and w(r) as in fmoe_combine,
+ *   d_value[r, :]          = round(dy[t, :] * w(r))
+ *   d_gates[flat(r)]       = sum_c round(value[r, c] * dy[t, c])      (fp32 sum; skipped if d_gates NULL)
+ * flat(r) = gates_index ? gates_index[r] : r.  value / dy / d_value share value_dtype.
+ */
+int fmoe_combine_bwd(const void* dy, const void* value, int value_dtype, int64_t T, int K, int64_t D,
+                     int64_t value_stride_row, const int64_t* token_index, const void* gates,
+                     int gates_dtype, int64_t gates_cols, int64_t gates_stride_row,
+                     int64_t gates_stride_col, const int64_t* gates_index, void* d_value,
+                     float* d_gates, fmoe_stream_t stream);
 
 #ifdef __cplusplus
 }

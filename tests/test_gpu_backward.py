@@ -1,0 +1,162 @@
+"""GPU parity of the backward pass: gradients of the HIP operators against torch autograd
+through the CPU oracle (fp32 accumulation), with the tolerances of the reference's own
+backward checks (kernels/tests/moe_test.py:276-297, 388-400)."""
+import pytest
+import torch
+
+from helpers import BF16, dev, make_routing, randn
+from oracle import layer as o_layer
+from oracle import moe as o_moe
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, ref, what, rtol=2e-2, atol_frac=1e-2):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    atol = atol_frac * ref.abs().max().item() + 1e-12
+    err = (got - ref).abs()
+    bad = err > atol + rtol * ref.abs()
+    assert not bad.any(), (f"{what}: {int(bad.sum())} of {bad.numel()} out of tolerance, max err "
+                           f"{err.max().item():.4g}, max |ref| {ref.abs().max().item():.4g}")
+
+
+def leaf(t, dtype=None, device=None):
+    t = t.detach().clone()
+    if dtype is not None:
+        t = t.to(dtype)
+    if device is not None:
+        t = t.to(device)
+    return t.requires_grad_(True)
+
+
+def kn_weight(E, K, N, seed, contiguous, scale):
+    w = randn((E, K, N), seed, scale=scale)
+    if not contiguous:
+        w = w.transpose(1, 2).contiguous().transpose(1, 2)
+    return w
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,contiguous", [
+    (100, 4, 2, 32, 32, True),
+    (500, 16, 4, 64, 128, False),
+    (2048, 8, 2, 256, 512, False),
+    (300, 8, 2, 40, 72, True),          # K / N tails, short experts
+])
+@pytest.mark.parametrize("dtype", [BF16, torch.float32])
+def test_index_select_jagged_bmm_backward(L, E, K, Din, Dout, contiguous, dtype):
+    from fast_moe_amd.kernels import moe
+    if dtype == torch.float32 and L > 600:
+        pytest.skip("fp32 grid kept small")
+    r = make_routing(L, E, K, seed=L + 1)
+    x0 = randn((L, Din), 1).to(dtype)
+    w0 = kn_weight(E, Din, Dout, 2, contiguous, Din ** -0.5).to(dtype)
+    b0 = randn((E, Dout), 3).to(dtype)
+    dout = (randn((L * K, Dout), 4) * 0.01).to(dtype)
+    xr, wr, br = leaf(x0, torch.float32), leaf(w0, torch.float32), leaf(b0, torch.float32)
+    o_moe.index_select_jagged_bmm(r["offsets"], r["index"], xr, wr, br).backward(dout.float())
+    x, w, b = leaf(x0, device="cuda"), leaf(w0, device="cuda"), leaf(b0, device="cuda")
+    out = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, b)
+    out.backward(dev(dout))
+    tol = dict(rtol=2e-2, atol_frac=1e-2) if dtype == BF16 else dict(rtol=1e-4, atol_frac=1e-5)
+    close(x.grad, xr.grad, "d_jagged", **tol)
+    close(w.grad, wr.grad, "d_weight", **tol)
+    close(b.grad, br.grad, "d_bias", **tol)
+    assert x.grad.dtype == dtype and w.grad.shape == w.shape
+
+
+@pytest.mark.parametrize("L,E,K,Din,H", [(256, 4, 2, 64, 96), (1024, 16, 4, 128, 192)])
+def test_swiglu_backward(L, E, K, Din, H):
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=7)
+    x0 = randn((L, Din), 1)
+    wg0, wu0 = kn_weight(E, Din, H, 2, False, Din ** -0.5), kn_weight(E, Din, H, 3, False, Din ** -0.5)
+    bg0, bu0 = randn((E, H), 4), randn((E, H), 5)
+    dout = randn((L * K, H), 6) * 0.01
+    ref = [leaf(t, torch.float32) for t in (x0, wg0, bg0, wu0, bu0)]
+    o_moe.index_select_jagged_bmm_swiglu(r["offsets"], r["index"], *ref).backward(dout.float())
+    got = [leaf(t, device="cuda") for t in (x0, wg0, bg0, wu0, bu0)]
+    out = moe.index_select_jagged_bmm_swiglu(0, dev(r["offsets"]), dev(r["index"]), *got)
+    out.backward(dev(dout))
+    for name, g, q in zip(("d_jagged", "d_weight", "d_bias", "d_weight_p", "d_bias_p"), got, ref):
+        close(g.grad, q.grad, name, rtol=3e-2, atol_frac=1.5e-2)
+
+
+@pytest.mark.parametrize("gate_dtype", [BF16, torch.float32])
+def test_mul_merge_k_add_backward(gate_dtype):
+    from fast_moe_amd.kernels import moe
+    T, E, K, D = 300, 8, 4, 96
+    r = make_routing(T, E, K, seed=11)
+    v0 = randn((T * K, D), 1)
+    g0 = torch.rand((T, K), generator=torch.Generator().manual_seed(2)).to(gate_dtype)
+    out_dtype = torch.promote_types(BF16, gate_dtype)
+    dy = (randn((T, D), 3) * 0.01).to(out_dtype)
+    vr, gr = leaf(v0), leaf(g0)
+    o_moe.mul_merge_k_add(r["token_index"], vr, K, gr, r["gate_index"]).backward(dy)
+    v, g = leaf(v0, device="cuda"), leaf(g0, device="cuda")
+    out = moe.mul_merge_k_add(dev(r["token_index"]), dev(r["reverse_index"]), v, weight=g,
+                              weight_index=dev(r["gate_index"]))
+    out.backward(dev(dy))
+    if gate_dtype == BF16:      # round(dy * w): the same single rounding as autograd's bf16 mul
+        assert torch.equal(v.grad.cpu(), vr.grad)
+    else:
+        close(v.grad, vr.grad, "d_value", rtol=1e-2, atol_frac=1e-3)
+    close(g.grad, gr.grad, "d_weight", rtol=1e-2, atol_frac=1e-2)
+
+
+@pytest.mark.parametrize("has_silu", [True, False])
+def test_silu_jagged_bmm_combine_backward(has_silu):
+    from fast_moe_amd.kernels import moe
+    T, E, K, H, O = 512, 8, 2, 96, 128
+    r = make_routing(T, E, K, seed=13)
+    j0 = randn((T * K, H), 1)
+    w0 = kn_weight(E, H, O, 2, False, H ** -0.5)
+    b0 = randn((E, O), 3)
+    g0 = torch.rand((T, K), generator=torch.Generator().manual_seed(4)).to(BF16)
+    dy = randn((T, O), 5) * 0.01
+    ref = [leaf(t, torch.float32) for t in (j0, w0, b0, g0)]
+    o_moe.silu_jagged_bmm_combine(r["offsets"], ref[0], ref[1], ref[2], r["token_index"], K, ref[3],
+                                  r["gate_index"], has_silu).backward(dy.float())
+    got = [leaf(t, device="cuda") for t in (j0, w0, b0, g0)]
+    out = moe.silu_jagged_bmm_combine(0, dev(r["offsets"]), got[0], got[1], got[2], dev(r["token_index"]),
+                                      dev(r["reverse_index"]), got[3], dev(r["gate_index"]), has_silu=has_silu)
+    out.backward(dev(dy))
+    for name, g, q in zip(("d_jagged", "d_weight", "d_bias", "d_gates"), got, ref):
+        close(g.grad, q.grad, name, rtol=3e-2, atol_frac=1.5e-2)
+
+
+def test_layer_backward_matches_oracle():
+    """FastMoELayer under grad mode: every parameter and the input receive the oracle's gradient."""
+    from fast_moe_amd import FastMoELayer
+    torch.manual_seed(0)
+    B, S, D, H, O, E, k = 2, 128, 64, 96, 64, 8, 2
+    layer = FastMoELayer(D, H, O, E, dtype=torch.float32)
+    with torch.no_grad():
+        layer._experts_hidden_bias.normal_(0, 0.1)
+        layer._experts_bias.normal_(0, 0.1)
+    x0 = torch.randn(B, S, D)
+    dy = torch.randn(B, S, O) * 0.01
+    params = {n: p.detach().clone().requires_grad_(True) for n, p in layer.named_parameters()}
+    xr = x0.clone().requires_grad_(True)
+    # oracle: the dense every-expert formulation is differentiable end to end
+    y_ref = o_layer.dense_moe_forward(xr, params["gate.gate.weight"], params["gate.gate.bias"],
+                                      params["_experts_hidden_w"], params["_experts_hidden_bias"],
+                                      params["_experts_w"], params["_experts_bias"], k)
+    y_ref.backward(dy)
+    layer = layer.cuda()
+    x = x0.cuda().requires_grad_(True)
+    y = layer(x, k)
+    torch.testing.assert_close(y.cpu(), y_ref.detach(), rtol=1e-4, atol=1e-5)
+    y.backward(dy.cuda())
+    close(x.grad, xr.grad, "d_x", rtol=1e-3, atol_frac=1e-4)
+    for n, p in layer.named_parameters():
+        close(p.grad, params[n].grad, n, rtol=1e-3, atol_frac=1e-4)
+
+
+def test_forward_only_operators_still_refuse_grad():
+    from fast_moe_amd.kernels import moe_fp8
+    r = make_routing(64, 4, 2, seed=1)
+    x = randn((64, 32), 1).cuda().requires_grad_(True)
+    w = randn((4, 32, 32), 2).cuda()
+    with pytest.raises(RuntimeError):
+        moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, None, fp8=True)
