@@ -276,6 +276,41 @@ def cpu_baseline(w, budget_s=12.0):
         sample_T *= 4
 
 
+def run_train(w, steps, warmup):
+    """Forward + backward of the SwiGLU MoE through the differentiable operators (bf16): the
+    training step of SURVEY 8(f).1, reported beside the forward metric, never instead of it."""
+    from fast_moe_amd.kernels import moe
+    from fast_moe_amd.kernels.hip import ops
+    dev = torch.device("cuda:0")
+    inp = make_inputs(w, dev)
+    T, K = w["T"], w["K"]
+    leaf = lambda t: t.detach().clone().requires_grad_(True)
+    x, wg, wu, wd = leaf(inp["x"]), leaf(inp["w_gate"]), leaf(inp["w_up"]), leaf(inp["w_down"])
+    dy = torch.randn(T, w["O"], device=dev).to(torch.bfloat16) * 0.01
+    stream = torch.cuda.current_stream(dev)
+
+    def forward():
+        r = ops.route_topk(inp["scores"], K)
+        gates = r["gates"].to(torch.bfloat16).requires_grad_(True)
+        h = moe.index_select_jagged_bmm_swiglu(0, r["offsets"], r["gate_index"].view(T, K), x,
+                                               wg.permute(0, 2, 1), None, wu.permute(0, 2, 1), None)
+        return moe.silu_jagged_bmm_combine(0, r["offsets"], h, wd.permute(0, 2, 1), None, r["token_index"],
+                                           r["reverse_index"], gates, r["gate_index"], has_silu=False)
+
+    def step():
+        for t in (x, wg, wu, wd):
+            t.grad = None
+        forward().backward(dy)
+
+    for _ in range(max(warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    ms = time_region(step, steps, stream)
+    ms_fwd = time_region(lambda: forward(), steps, stream)
+    f1, f2 = flops_of(w)
+    return ms, ms_fwd, 3.0 * (f1 + f2)
+
+
 def bench_workload(name, steps, warmup, tokens=None):
     w = dict(WORKLOADS[name])
     if tokens:
@@ -293,6 +328,8 @@ def main():
     ap.add_argument("--tokens", type=int, default=None, help="override the token count (C5 sweep)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary fp8 / bf16 workload")
+    ap.add_argument("--backward", action="store_true",
+                    help="time forward + backward of the bf16 SwiGLU workload instead of the forward metric")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 512 MiB device copy, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -304,6 +341,23 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
 
+    if args.backward:
+        w = dict(WORKLOADS[args.workload])
+        if w["kind"] != "swiglu" or w["dtype"] != "bf16":
+            print("bench.py --backward: a bf16 swiglu workload is required", file=sys.stderr)
+            sys.exit(2)
+        if args.tokens:
+            w["T"] = args.tokens
+        ms, ms_fwd, flops = run_train(w, args.steps, args.warmup)
+        print(json.dumps({
+            "metric": "moe_fwd_bwd_tflops", "value": round(flops / ms / 1e9, 2), "unit": "TFLOP/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4),
+            "ms_forward_with_saved_tensors": round(ms_fwd, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"{args.workload}: swiglu MoE forward + backward (input, weight and gate "
+                                   f"gradients), T={w['T']}, E={w['E']}, top-{w['K']}, D={w['D']}, H={w['H']}",
+                       "flops": "3 x forward GEMM FLOPs"}}))
+        return
     w, ms, kernels, stats, flops = bench_workload(args.workload, args.steps, args.warmup, args.tokens)
     dt = w["dtype"]
     g1 = kernels["gemm1"]

@@ -305,14 +305,25 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_kernel(const GemmParams p
     const int64_t total_tiles = total_m * p.n_tiles;
     const int64_t per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
     const int64_t slot = blockIdx.x / kNumXcd;
-    if (slot >= per_xcd) return;
-    const int64_t logical = (int64_t)(blockIdx.x % kNumXcd) * per_xcd + slot;
-    if (logical >= total_tiles) return;
     const int64_t group_span = (int64_t)kGroupM * p.n_tiles;
-    const int64_t group = logical / group_span;
+    int64_t group;
+    int within;
+    if (p.k_window) {
+        // the cost of a tile follows its expert's contraction length, so contiguous tile ranges
+        // per XCD would leave one XCD with the long experts: deal the groups out round-robin
+        group = slot / group_span * kNumXcd + blockIdx.x % kNumXcd;
+        within = (int)(slot % group_span);
+    } else {
+        if (slot >= per_xcd) return;
+        const int64_t logical = (int64_t)(blockIdx.x % kNumXcd) * per_xcd + slot;
+        if (logical >= total_tiles) return;
+        group = logical / group_span;
+        within = (int)(logical - group * group_span);
+    }
     const int64_t first_m = group * kGroupM;
+    if (first_m >= total_m) return;
     const int gsize = (int)(total_m - first_m < kGroupM ? total_m - first_m : kGroupM);
-    const int within = (int)(logical - group * group_span);
+    if (within >= gsize * p.n_tiles) return;
     const int64_t mt = first_m + within % gsize;
     const int nt = within / gsize;
 
@@ -1211,7 +1222,11 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
     if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
     const int64_t max_m_tiles = p.total_rows / TL::BM + p.E;
     const int64_t max_tiles = max_m_tiles * p.n_tiles;
-    const int64_t grid = (max_tiles + kNumXcd - 1) / kNumXcd * kNumXcd;
+    int64_t grid = (max_tiles + kNumXcd - 1) / kNumXcd * kNumXcd;
+    if (p.k_window) {      // whole groups of kGroupM row tiles per XCD, round-robin
+        const int64_t groups = (max_m_tiles + kGroupM - 1) / kGroupM;
+        grid = (groups + kNumXcd - 1) / kNumXcd * kNumXcd * kGroupM * p.n_tiles;
+    }
     if (grid >= ((int64_t)1 << 31)) return fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: grid too large");
     kern<<<(unsigned)grid, TL::NT, TL::LDS_BYTES, stream>>>(p);
     return check_launch("fmoe_grouped_gemm");

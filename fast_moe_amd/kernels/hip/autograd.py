@@ -69,11 +69,14 @@ def weight_grad(a_src: torch.Tensor, dout: torch.Tensor, offsets: torch.Tensor, 
 def _input_grad(drow_list, weights, offsets, reverse_index) -> torch.Tensor:
     """sum over branches and over the K rows of a token of drow @ W^T -> [T, K_in]."""
     R = drow_list[0].shape[0]
-    parts = [ops.grouped_gemm(offsets, d, w.permute(0, 2, 1), total_rows=R) for d, w in zip(drow_list, weights)]
-    if len(parts) == 1:
-        return ops.combine(parts[0], reverse_index)
-    value = torch.cat(parts, dim=0)
-    rev = torch.cat([reverse_index + i * R for i in range(len(parts))], dim=1)
+    n = len(drow_list)
+    Kin = weights[0].shape[1]
+    value = torch.empty((n * R, Kin), dtype=drow_list[0].dtype, device=drow_list[0].device)
+    for i, (d, w) in enumerate(zip(drow_list, weights)):
+        ops.grouped_gemm(offsets, d, w.permute(0, 2, 1), total_rows=R, out=value[i * R:(i + 1) * R])
+    if n == 1:
+        return ops.combine(value, reverse_index)
+    rev = torch.cat([reverse_index + i * R for i in range(n)], dim=1)
     return ops.combine(value, rev)
 
 

@@ -181,7 +181,7 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  bias2: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE, a_silu: bool = False,
                  a_scale: Optional[torch.Tensor] = None, b_scale: Optional[torch.Tensor] = None,
                  b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0,
-                 k_window: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 k_window: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
     strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
     [total_rows, N] in bf16 (fp32 for fp32 operands)."""
@@ -220,7 +220,11 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
         row_index = _i64("row_index", row_index).view(-1)
         if row_index.numel() != total_rows:
             raise ValueError("grouped_gemm: row_index must have total_rows entries")
-    out = torch.empty((total_rows, N), dtype=out_dtype, device=dev)
+    if out is None:
+        out = torch.empty((total_rows, N), dtype=out_dtype, device=dev)
+    elif (tuple(out.shape) != (total_rows, N) or out.dtype != out_dtype or out.device != dev
+          or out.stride(1) != 1):
+        raise ValueError(f"grouped_gemm: out must be {out_dtype} [{total_rows}, {N}] with contiguous rows")
     if total_rows == 0:
         return out
 
