@@ -69,6 +69,85 @@ __global__ __launch_bounds__(256) void jagged_transpose_kernel(
     }
 }
 
+// bf16 fast path: 64 (padded rows) x 128 (columns) tile.  Source rows come in with 16-byte
+// loads and go to LDS row-major; ds_read_b64_tr_b16 reads them back transposed (within 16
+// lanes, lane j receives element j of 4 consecutive rows when lane i points at row i/4,
+// elements 4*(i%4)..+3), so two such reads give a lane 8 consecutive padded rows of one
+// column: one 16-byte store.  LDS rows are 320 bytes apart: the four rows of a 16-lane group
+// and the two groups served in one pass then fall into eight different 32-byte bank groups.
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__global__ __launch_bounds__(256) void jagged_transpose_tr_kernel(
+    const uint16_t* __restrict__ src, int64_t src_rows, int64_t cols, int64_t src_stride,
+    const int64_t* __restrict__ row_index, int index_div, const int64_t* __restrict__ offsets,
+    const int64_t* __restrict__ pad_offsets, int E, uint16_t* __restrict__ dst, int64_t dst_stride,
+    int64_t dst_cols, int apply_silu) {
+    constexpr int ROWB = 320;
+    __shared__ __align__(16) uint8_t tile[64 * ROWB];
+    __shared__ int64_t s_src[64];
+    const int64_t p0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 128;
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+        const int64_t pcol = p0 + tid;
+        int64_t srow = -1;
+        if (pcol < pad_offsets[E]) {
+            int lo = 0, hi = E;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (pad_offsets[mid] <= pcol) lo = mid; else hi = mid;
+            }
+            const int64_t j = pcol - pad_offsets[lo];
+            const int64_t len = offsets[lo + 1] - offsets[lo];
+            if (j >= 0 && j < len) {
+                int64_t r = offsets[lo] + j;
+                if (row_index) r = row_index[r] / index_div;
+                if (r >= 0 && r < src_rows) srow = r;
+            }
+        }
+        s_src[tid] = srow;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = (tid >> 4) + 16 * i, chunk = tid & 15;
+        const int64_t r = s_src[row], c = c0 + chunk * 8;
+        u32x4 v = {0, 0, 0, 0};
+        if (r >= 0 && c < cols) {          // cols is a multiple of 8 on this path
+            v = *reinterpret_cast<const u32x4*>(src + r * src_stride + c);
+            if (apply_silu) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float lo = silu_f32(bf16_bits_to_f32(v[q] & 0xffffu));
+                    const float hi = silu_f32(__uint_as_float(v[q] & 0xffff0000u));
+                    v[q] = f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+                }
+            }
+        }
+        *reinterpret_cast<u32x4*>(tile + row * ROWB + chunk * 16) = v;
+    }
+    __syncthreads();
+    const int lane = tid & 63, wave = tid >> 6;
+    const int grp = lane >> 4, j = lane & 15;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int pb = 2 * wave + (it & 1), half = it >> 1;
+        const int cbase = 64 * half + 16 * grp;
+        // this lane's read address: row 8*pb + j/4 (+4 for the second read), columns cbase + 4*(j%4)..+3
+        uint8_t* a = tile + (8 * pb + (j >> 2)) * ROWB + (cbase + 4 * (j & 3)) * 2;
+        typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)a);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(a + 4 * ROWB));
+        const int64_t c = c0 + cbase + j, pcol = p0 + 8 * pb;
+        if (c < cols && pcol < dst_cols) {   // dst_cols is a multiple of 8 on this path
+            u32x4 o;
+            o[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+            o[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+            o[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+            o[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+            *reinterpret_cast<u32x4*>(dst + c * dst_stride + pcol) = o;
+        }
+    }
+}
+
 // one block per (expert, 64 columns): 4 row lanes add every 4th row, then a fixed-order tree
 template <typename T>
 __global__ __launch_bounds__(256) void segment_colsum_kernel(const T* __restrict__ src, int64_t total_rows,
@@ -178,7 +257,15 @@ extern "C" int fmoe_jagged_transpose(const void* src, int dtype, int64_t src_row
     const int64_t gx = (dst_cols + 63) / 64, gy = (cols + 63) / 64;
     FMOE_REQUIRE(gx < ((int64_t)1 << 31) && gy <= 65535, "fmoe_jagged_transpose: grid too large");
     dim3 grid((unsigned)gx, (unsigned)gy);
-    if (dtype == FMOE_BF16)
+    const bool vec = dtype == FMOE_BF16 && cols % 8 == 0 && src_stride_row % 8 == 0 && dst_stride % 8 == 0 &&
+                     dst_cols % 8 == 0 && aligned16(src) && aligned16(dst);
+    if (vec) {
+        const int64_t gy2 = (cols + 127) / 128;
+        dim3 grid2((unsigned)gx, (unsigned)gy2);
+        jagged_transpose_tr_kernel<<<grid2, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, src_rows, cols, src_stride_row, row_index, index_div, offsets, pad_offsets,
+            num_experts, (uint16_t*)dst, dst_stride, dst_cols, apply_silu);
+    } else if (dtype == FMOE_BF16)
         jagged_transpose_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
             (const uint16_t*)src, src_rows, cols, src_stride_row, row_index, index_div, offsets, pad_offsets,
             num_experts, (uint16_t*)dst, dst_stride, dst_cols, apply_silu);

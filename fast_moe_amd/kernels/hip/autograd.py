@@ -46,24 +46,31 @@ def _reverse_from_index(index: torch.Tensor) -> torch.Tensor:
     return inv.view(T, K).sort(dim=1).values
 
 
-def weight_grad(a_src: torch.Tensor, dout: torch.Tensor, offsets: torch.Tensor, *,
-                row_index: Optional[torch.Tensor] = None, index_div: int = 1,
-                apply_silu: bool = False) -> torch.Tensor:
-    """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a(r)[k], a(r) = the (gathered,
-    optionally SiLU-ed) input row of routed row r.  Returns [E, N, K] contiguous."""
-    R, N = dout.shape
-    Kin = a_src.shape[1]
-    E = offsets.numel() - 1
-    pad_offsets, bound = _pad_layout(offsets, R)
-    dout_t = ops.jagged_transpose(dout, offsets, pad_offsets, bound)                       # [N, bound]
-    a_t = ops.jagged_transpose(a_src, offsets, pad_offsets, bound, row_index, index_div, apply_silu)  # [Kin, bound]
-    dev = dout.device
-    seg = torch.arange(E + 1, device=dev, dtype=torch.int64) * N
-    rows = torch.arange(E * N, device=dev, dtype=torch.int64) % N
-    b = a_t.t().unsqueeze(0).expand(E, bound, Kin)                                          # B[e, k, n'] = a_t[n', k]
-    dw = ops.grouped_gemm(seg, dout_t, b, total_rows=E * N, row_index=rows, index_div=1, epilogue=EPI_NONE,
-                          k_window=pad_offsets)
-    return dw.view(E, N, Kin)
+class _WgradOperand:
+    """The input rows of the routed rows, transposed and zero padded per expert ([K_in, bound]),
+    with the padded layout it was written in: shared by the weight gradients of every weight
+    that multiplied the same input (SwiGLU's gate and up projections)."""
+
+    def __init__(self, a_src: torch.Tensor, offsets: torch.Tensor, total_rows: int, *,
+                 row_index: Optional[torch.Tensor] = None, index_div: int = 1, apply_silu: bool = False):
+        self.offsets = offsets
+        self.pad_offsets, self.bound = _pad_layout(offsets, total_rows)
+        self.a_t = ops.jagged_transpose(a_src, offsets, self.pad_offsets, self.bound, row_index, index_div,
+                                        apply_silu)
+
+    def weight_grad(self, dout: torch.Tensor) -> torch.Tensor:
+        """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a(r)[k] -> [E, N, K_in]."""
+        N = dout.shape[1]
+        Kin = self.a_t.shape[0]
+        E = self.offsets.numel() - 1
+        dout_t = ops.jagged_transpose(dout, self.offsets, self.pad_offsets, self.bound)        # [N, bound]
+        dev = dout.device
+        seg = torch.arange(E + 1, device=dev, dtype=torch.int64) * N
+        rows = torch.arange(E * N, device=dev, dtype=torch.int64) % N
+        b = self.a_t.t().unsqueeze(0).expand(E, self.bound, Kin)                               # B[e, k, n'] = a_t[n', k]
+        dw = ops.grouped_gemm(seg, dout_t, b, total_rows=E * N, row_index=rows, index_div=1, epilogue=EPI_NONE,
+                              k_window=self.pad_offsets)
+        return dw.view(E, N, Kin)
 
 
 def _input_grad(drow_list, weights, offsets, reverse_index) -> torch.Tensor:
@@ -111,13 +118,15 @@ class IndexSelectJaggedBmm(torch.autograd.Function):
         d_jagged = d_w = d_b = d_wp = d_bp = None
         if need[2]:
             d_jagged = _input_grad(drows, weights, offsets, _reverse_from_index(index)).view_as(jagged)
-        flat_index = index.reshape(-1)
+        operand = None
+        if need[3] or (swiglu and need[5]):
+            operand = _WgradOperand(jagged, offsets, R, row_index=index.reshape(-1), index_div=K)
         if need[3]:
-            d_w = weight_grad(jagged, drows[0], offsets, row_index=flat_index, index_div=K).permute(0, 2, 1)
+            d_w = operand.weight_grad(drows[0]).permute(0, 2, 1)
         if bias is not None and need[4]:
             d_b = ops.segment_colsum(drows[0], offsets)
         if swiglu and need[5]:
-            d_wp = weight_grad(jagged, drows[1], offsets, row_index=flat_index, index_div=K).permute(0, 2, 1)
+            d_wp = operand.weight_grad(drows[1]).permute(0, 2, 1)
         if swiglu and bias_p is not None and need[6]:
             d_bp = ops.segment_colsum(drows[1], offsets)
         return None, None, d_jagged, d_w, d_b, d_wp, d_bp
@@ -169,7 +178,8 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
             d_h = ops.grouped_gemm(offsets, d_bmm, weight.permute(0, 2, 1), total_rows=d_bmm.shape[0])
             d_jagged = ops.swiglu_bwd(jagged, None, d_h)[0] if ctx.has_silu else d_h
         if need[2]:
-            d_w = weight_grad(jagged, d_bmm, offsets, apply_silu=ctx.has_silu).permute(0, 2, 1)
+            operand = _WgradOperand(jagged, offsets, jagged.shape[0], apply_silu=ctx.has_silu)
+            d_w = operand.weight_grad(d_bmm).permute(0, 2, 1)
         if bias is not None and need[3]:
             d_b = ops.segment_colsum(d_bmm, offsets)
         if need_g:

