@@ -192,6 +192,43 @@ __global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ g
     }
 }
 
+// bf16, 8 elements per thread (16-byte loads and stores)
+template <bool GATED>
+__global__ __launch_bounds__(256) void swiglu_bwd_bf16x8_kernel(const uint16_t* __restrict__ g,
+                                                                const uint16_t* __restrict__ u,
+                                                                const uint16_t* __restrict__ dh,
+                                                                uint16_t* __restrict__ dg,
+                                                                uint16_t* __restrict__ du, int64_t n8) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const u32x4 vg = reinterpret_cast<const u32x4*>(g)[i];
+    const u32x4 vd = reinterpret_cast<const u32x4*>(dh)[i];
+    u32x4 vu = {0, 0, 0, 0}, og, ou = {0, 0, 0, 0};
+    if (GATED) vu = reinterpret_cast<const u32x4*>(u)[i];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        uint32_t rg = 0, ru = 0;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const float gv = bf16_bits_to_f32((vg[q] >> (16 * h)) & 0xffffu);
+            const float d = bf16_bits_to_f32((vd[q] >> (16 * h)) & 0xffffu);
+            const float s = sigmoid_f32(gv);
+            const float dsilu = s * (1.0f + gv * (1.0f - s));
+            if (GATED) {
+                const float uv = bf16_bits_to_f32((vu[q] >> (16 * h)) & 0xffffu);
+                ru |= f32_to_bf16_bits(d * round_bf16(gv * s)) << (16 * h);
+                rg |= f32_to_bf16_bits(round_bf16(d * uv) * dsilu) << (16 * h);
+            } else {
+                rg |= f32_to_bf16_bits(d * dsilu) << (16 * h);
+            }
+        }
+        og[q] = rg;
+        ou[q] = ru;
+    }
+    reinterpret_cast<u32x4*>(dg)[i] = og;
+    if (GATED) reinterpret_cast<u32x4*>(du)[i] = ou;
+}
+
 struct GateArgs {
     const void* ptr;
     int64_t cols, stride_row, stride_col;
@@ -206,7 +243,7 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ 
                                                           int64_t value_stride,
                                                           const int64_t* __restrict__ token_index,
                                                           GateArgs gate, T* __restrict__ d_value,
-                                                          float* __restrict__ d_gates) {
+                                                          float* __restrict__ d_gates, bool vec8) {
     const int lane = lane_id();
     const int64_t r = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
     if (r >= R) return;
@@ -224,10 +261,31 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ 
         }
     }
     float dot = 0.0f;
-    for (int64_t c = lane; c < D; c += kWave) {
-        const float d = ok ? Val<T>::load(dy + t * D + c) : 0.0f;
-        Val<T>::store(d_value + r * D + c, d * w);
-        if (d_gates) dot += Val<T>::round(Val<T>::load(value + r * value_stride + c) * d);
+    if (sizeof(T) == 2 && vec8) {
+        const uint16_t* dyr = (const uint16_t*)dy + t * D;
+        const uint16_t* vr = (const uint16_t*)value + r * value_stride;
+        uint16_t* dvr = (uint16_t*)d_value + r * D;
+        for (int64_t c = (int64_t)lane * 8; c < D; c += kWave * 8) {
+            u32x4 vd = {0, 0, 0, 0}, vv = {0, 0, 0, 0}, o;
+            if (ok) vd = *reinterpret_cast<const u32x4*>(dyr + c);
+            if (d_gates) vv = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vr + c));
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float d0 = bf16_bits_to_f32(vd[q] & 0xffffu), d1 = __uint_as_float(vd[q] & 0xffff0000u);
+                o[q] = f32_to_bf16_bits(d0 * w) | (f32_to_bf16_bits(d1 * w) << 16);
+                if (d_gates) {
+                    dot += round_bf16(bf16_bits_to_f32(vv[q] & 0xffffu) * d0);
+                    dot += round_bf16(__uint_as_float(vv[q] & 0xffff0000u) * d1);
+                }
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(dvr + c));
+        }
+    } else {
+        for (int64_t c = lane; c < D; c += kWave) {
+            const float d = ok ? Val<T>::load(dy + t * D + c) : 0.0f;
+            Val<T>::store(d_value + r * D + c, d * w);
+            if (d_gates) dot += Val<T>::round(Val<T>::load(value + r * value_stride + c) * d);
+        }
     }
     if (d_gates) {
 #pragma unroll
@@ -304,7 +362,13 @@ extern "C" int fmoe_swiglu_bwd(const void* g, const void* u, const void* dh, voi
     const unsigned blocks = (unsigned)((n + 255) / 256);
     FMOE_REQUIRE((n + 255) / 256 < ((int64_t)1 << 31), "fmoe_swiglu_bwd: too many elements");
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == FMOE_BF16) {
+    if (dtype == FMOE_BF16 && n % 8 == 0 && aligned16(g) && aligned16(dh) && aligned16(dg) &&
+        (!u || (aligned16(u) && aligned16(du)))) {
+        const int64_t n8 = n / 8;
+        const unsigned b8 = (unsigned)((n8 + 255) / 256);
+        if (u) swiglu_bwd_bf16x8_kernel<true><<<b8, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)u, (const uint16_t*)dh, (uint16_t*)dg, (uint16_t*)du, n8);
+        else swiglu_bwd_bf16x8_kernel<false><<<b8, 256, 0, s>>>((const uint16_t*)g, nullptr, (const uint16_t*)dh, (uint16_t*)dg, nullptr, n8);
+    } else if (dtype == FMOE_BF16) {
         if (u) swiglu_bwd_kernel<uint16_t, true><<<blocks, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)u, (const uint16_t*)dh, (uint16_t*)dg, (uint16_t*)du, n);
         else swiglu_bwd_kernel<uint16_t, false><<<blocks, 256, 0, s>>>((const uint16_t*)g, nullptr, (const uint16_t*)dh, (uint16_t*)dg, nullptr, n);
     } else {
@@ -334,12 +398,14 @@ extern "C" int fmoe_combine_bwd(const void* dy, const void* value, int value_dty
     const unsigned blocks = (unsigned)((R + 3) / 4);
     hipStream_t s = (hipStream_t)stream;
     const bool gb = gates && gates_dtype == FMOE_BF16;
+    const bool vec8 = D % 8 == 0 && aligned16(dy) && aligned16(d_value) &&
+                      (!d_gates || (value_stride_row % 8 == 0 && aligned16(value)));
     if (value_dtype == FMOE_BF16) {
-        if (gb) combine_bwd_kernel<uint16_t, uint16_t><<<blocks, 256, 0, s>>>((const uint16_t*)dy, (const uint16_t*)value, T, R, D, value_stride_row, token_index, ga, (uint16_t*)d_value, d_gates);
-        else combine_bwd_kernel<uint16_t, float><<<blocks, 256, 0, s>>>((const uint16_t*)dy, (const uint16_t*)value, T, R, D, value_stride_row, token_index, ga, (uint16_t*)d_value, d_gates);
+        if (gb) combine_bwd_kernel<uint16_t, uint16_t><<<blocks, 256, 0, s>>>((const uint16_t*)dy, (const uint16_t*)value, T, R, D, value_stride_row, token_index, ga, (uint16_t*)d_value, d_gates, vec8);
+        else combine_bwd_kernel<uint16_t, float><<<blocks, 256, 0, s>>>((const uint16_t*)dy, (const uint16_t*)value, T, R, D, value_stride_row, token_index, ga, (uint16_t*)d_value, d_gates, vec8);
     } else {
-        if (gb) combine_bwd_kernel<float, uint16_t><<<blocks, 256, 0, s>>>((const float*)dy, (const float*)value, T, R, D, value_stride_row, token_index, ga, (float*)d_value, d_gates);
-        else combine_bwd_kernel<float, float><<<blocks, 256, 0, s>>>((const float*)dy, (const float*)value, T, R, D, value_stride_row, token_index, ga, (float*)d_value, d_gates);
+        if (gb) combine_bwd_kernel<float, uint16_t><<<blocks, 256, 0, s>>>((const float*)dy, (const float*)value, T, R, D, value_stride_row, token_index, ga, (float*)d_value, d_gates, false);
+        else combine_bwd_kernel<float, float><<<blocks, 256, 0, s>>>((const float*)dy, (const float*)value, T, R, D, value_stride_row, token_index, ga, (float*)d_value, d_gates, false);
     }
     return check_launch("fmoe_combine_bwd");
 }
