@@ -100,6 +100,17 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert lib.fmoe_combine(ctypes.c_void_p(64), 1, 4, 2, 8, 8, ctypes.c_void_p(64), ctypes.c_void_p(64), 0, 2,
                             2, 1, None, ctypes.c_void_p(64), 1, None) == 1
     assert b"promoted" in lib.fmoe_last_error()
+    # backward helpers: dtype and stride checks come before any launch
+    P = ctypes.c_void_p(64)
+    assert lib.fmoe_jagged_transpose(P, 2, 8, 8, 8, None, 1, P, P, 2, P, 16, 16, 0, None) == 1
+    assert b"bf16 or fp32" in lib.fmoe_last_error()
+    assert lib.fmoe_jagged_transpose(P, 1, 8, 8, 4, None, 1, P, P, 2, P, 16, 16, 0, None) == 1
+    assert b"row stride" in lib.fmoe_last_error()
+    assert lib.fmoe_segment_colsum(P, 1, 8, 8, 4, P, 2, P, None) == 1
+    assert lib.fmoe_swiglu_bwd(P, P, P, P, None, 1, 8, None) == 1          # gated form needs du
+    assert lib.fmoe_combine_bwd(P, None, 1, 4, 2, 8, 8, P, None, 0, 1, 1, 1, None, P,
+                                ctypes.cast(P, ctypes.POINTER(ctypes.c_float)), None) == 1
+    assert b"d_gates needs value" in lib.fmoe_last_error()
 
 
 def test_pytorch_kernel_is_refused():
