@@ -135,26 +135,33 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         rsa[fm] = 1.0f;
         if (FP8) rsa[fm] = 1.0f / p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))];
     }
+    // per-column epilogue constants of this lane: [fn][gp][q][j] <-> column nq + 8*q + 4*khalf + j
+    // with nq = first column of register-quad pair gp of fragment fn
+    float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
+    const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
 #pragma unroll
-    for (int fn = 0; fn < FN_OUT; ++fn) {
+    for (int fn = 0; fn < FN_OUT; ++fn)
 #pragma unroll
-        for (int gp = 0; gp < 2; ++gp) {
-            // register quads g = 2gp and 2gp+1: columns nq + 8*q + 4*khalf + j
-            const int nq = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN) + fn * 32 + 16 * gp;
-            float rsw[2][4], rsw2[2][4], bv[2][4], bv2[2][4];
+        for (int gp = 0; gp < 2; ++gp)
 #pragma unroll
             for (int q = 0; q < 2; ++q)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int n = nq + 8 * q + 4 * khalf + j;
+                    const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
                     const int nc = n < p.N ? n : p.N - 1;
-                    rsw[q][j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                    rsw2[q][j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                    bv[q][j] = p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
-                    bv2[q][j] = (SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
+                    rsw[fn][gp][q][j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                    rsw2[fn][gp][q][j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                    bv[fn][gp][q][j] = p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
+                    bv2[fn][gp][q][j] = (SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
                 }
+    // rows outermost: the stores that complete a row's 128-byte line follow each other
 #pragma unroll
-            for (int fm = 0; fm < FM; ++fm) {
+    for (int fm = 0; fm < FM; ++fm) {
+#pragma unroll
+        for (int fn = 0; fn < FN_OUT; ++fn) {
+#pragma unroll
+            for (int gp = 0; gp < 2; ++gp) {
+                const int nq = col0 + fn * 32 + 16 * gp;
                 float o[2][4];
 #pragma unroll
                 for (int q = 0; q < 2; ++q)
@@ -164,15 +171,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         float y = acc[fn][fm][v];
                         float y2 = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
                         if (FP8) {
-                            y = rbf(y * (rsa[fm] * rsw[q][j]));
-                            if (p.bias) y = rbf(y + bv[q][j]);
+                            y = rbf(y * (rsa[fm] * rsw[fn][gp][q][j]));
+                            if (p.bias) y = rbf(y + bv[fn][gp][q][j]);
                             if (SWIGLU) {
-                                y2 = rbf(y2 * (rsa[fm] * rsw2[q][j]));
-                                if (p.bias2) y2 = rbf(y2 + bv2[q][j]);
+                                y2 = rbf(y2 * (rsa[fm] * rsw2[fn][gp][q][j]));
+                                if (p.bias2) y2 = rbf(y2 + bv2[fn][gp][q][j]);
                             }
                         } else {
-                            y = rbf(y + bv[q][j]);
-                            if (SWIGLU) y2 = rbf(y2 + bv2[q][j]);
+                            y = rbf(y + bv[fn][gp][q][j]);
+                            if (SWIGLU) y2 = rbf(y2 + bv2[fn][gp][q][j]);
                         }
                         if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
                         if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
