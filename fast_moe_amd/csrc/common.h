@@ -12,7 +12,6 @@
 namespace fmoe {
 
 // ---------------------------------------------------------------- host side
-void set_error(const char* fmt, ...);
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
 

@@ -7,13 +7,6 @@ namespace fmoe {
 
 static thread_local char g_error[512] = "";
 
-void set_error(const char* fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_error, sizeof(g_error), fmt, ap);
-    va_end(ap);
-}
-
 int fail(int code, const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);

@@ -919,9 +919,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     // vmcnt bookkeeping.  Loads return in order, so "at most n operations outstanding"
     // means everything but the n youngest operations has landed; stores or other loads in
     // the queue only make the wait longer, never shorter.
-    int landed = -1;                        // items <= landed are complete for this wave
-    int c = 0;                              // item being computed
-    int cslot = 0;                          // c % STAGES
+    int landed = -1;                        // 4-slot ring: items <= landed are complete for this wave
+    int c = 0;                              // 4-slot ring: item being computed
+    int cslot = 0;                          // ring slot of the item being computed
     bf16x8 wfa[FN], xfa[FM], wfb[FN], xfb[FM];   // fragment double buffer of the pipelined loop
     i32x8 qwa[FN], qwb[FN], qx0[FM / 2], qx1[FM / 2];   // the same for e4m3 fragments
     for (int tile_i = 0; tile_i < my_tiles; ++tile_i) {
