@@ -135,78 +135,84 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         rsa[fm] = 1.0f;
         if (FP8) rsa[fm] = 1.0f / p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))];
     }
-    // per-column epilogue constants of this lane: [fn][gp][q][j] <-> column nq + 8*q + 4*khalf + j
-    // with nq = first column of register-quad pair gp of fragment fn
-    float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
-    const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
+    // the bias-free form (FastMoE's SwiGLU experts, every fp8 call without bias) skips the adds
+    auto run = [&](auto has_bias_c) {
+        constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
+        // per-column epilogue constants of this lane: [fn][gp][q][j] <-> column nq + 8*q + 4*khalf + j
+        // with nq = first column of register-quad pair gp of fragment fn
+        float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
+        const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
 #pragma unroll
-    for (int fn = 0; fn < FN_OUT; ++fn)
+        for (int fn = 0; fn < FN_OUT; ++fn)
 #pragma unroll
-        for (int gp = 0; gp < 2; ++gp)
-#pragma unroll
-            for (int q = 0; q < 2; ++q)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
-                    const int nc = n < p.N ? n : p.N - 1;
-                    rsw[fn][gp][q][j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                    rsw2[fn][gp][q][j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                    bv[fn][gp][q][j] = p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
-                    bv2[fn][gp][q][j] = (SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
-                }
-    // rows outermost: the stores that complete a row's 128-byte line follow each other
-#pragma unroll
-    for (int fm = 0; fm < FM; ++fm) {
-#pragma unroll
-        for (int fn = 0; fn < FN_OUT; ++fn) {
-#pragma unroll
-            for (int gp = 0; gp < 2; ++gp) {
-                const int nq = col0 + fn * 32 + 16 * gp;
-                float o[2][4];
+            for (int gp = 0; gp < 2; ++gp)
 #pragma unroll
                 for (int q = 0; q < 2; ++q)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const int v = 4 * (2 * gp + q) + j;
-                        float y = acc[fn][fm][v];
-                        float y2 = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
-                        if (FP8) {
-                            y = rbf(y * (rsa[fm] * rsw[fn][gp][q][j]));
-                            if (p.bias) y = rbf(y + bv[fn][gp][q][j]);
-                            if (SWIGLU) {
-                                y2 = rbf(y2 * (rsa[fm] * rsw2[fn][gp][q][j]));
-                                if (p.bias2) y2 = rbf(y2 + bv2[fn][gp][q][j]);
-                            }
-                        } else {
-                            y = rbf(y + bv[fn][gp][q][j]);
-                            if (SWIGLU) y2 = rbf(y2 + bv2[fn][gp][q][j]);
-                        }
-                        if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
-                        if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
-                        o[q][j] = y;
+                        const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
+                        const int nc = n < p.N ? n : p.N - 1;
+                        rsw[fn][gp][q][j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                        rsw2[fn][gp][q][j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                        bv[fn][gp][q][j] = HAS_BIAS && p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
+                        bv2[fn][gp][q][j] = (HAS_BIAS && SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
                     }
-                if (p.vec_store) {
-                    // pair the quads of the two lane halves: low lanes end up with columns
-                    // nq..nq+7, high lanes with nq+8..nq+15 of their row
-                    const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][0], o[0][1]),
-                                                                      pack_bf16(o[1][0], o[1][1]), false, false);
-                    const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][2], o[0][3]),
-                                                                      pack_bf16(o[1][2], o[1][3]), false, false);
-                    const int nb = nq + 8 * khalf;
-                    if (row_ok[fm] && nb + 7 < p.N)
-                        *reinterpret_cast<u32x4*>(orow[fm] + nb) = u32x4{s0[0], s1[0], s0[1], s1[1]};
-                } else if (row_ok[fm]) {
+        // rows outermost: the stores that complete a row's 128-byte line follow each other
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+#pragma unroll
+            for (int fn = 0; fn < FN_OUT; ++fn) {
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp) {
+                    const int nq = col0 + fn * 32 + 16 * gp;
+                    float o[2][4];
 #pragma unroll
                     for (int q = 0; q < 2; ++q)
 #pragma unroll
                         for (int j = 0; j < 4; ++j) {
-                            const int n = nq + 8 * q + 4 * khalf + j;
-                            if (n < p.N) orow[fm][n] = (uint16_t)f32_to_bf16_bits(o[q][j]);
+                            const int v = 4 * (2 * gp + q) + j;
+                            float y = acc[fn][fm][v];
+                            float y2 = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
+                            if (FP8) {
+                                y = rbf(y * (rsa[fm] * rsw[fn][gp][q][j]));
+                                if (HAS_BIAS && p.bias) y = rbf(y + bv[fn][gp][q][j]);
+                                if (SWIGLU) {
+                                    y2 = rbf(y2 * (rsa[fm] * rsw2[fn][gp][q][j]));
+                                    if (HAS_BIAS && p.bias2) y2 = rbf(y2 + bv2[fn][gp][q][j]);
+                                }
+                            } else {
+                                y = rbf(HAS_BIAS ? y + bv[fn][gp][q][j] : y);
+                                if (SWIGLU) y2 = rbf(HAS_BIAS ? y2 + bv2[fn][gp][q][j] : y2);
+                            }
+                            if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
+                            if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
+                            o[q][j] = y;
                         }
+                    if (p.vec_store) {
+                        // pair the quads of the two lane halves: low lanes end up with columns
+                        // nq..nq+7, high lanes with nq+8..nq+15 of their row
+                        const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][0], o[0][1]),
+                                                                          pack_bf16(o[1][0], o[1][1]), false, false);
+                        const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][2], o[0][3]),
+                                                                          pack_bf16(o[1][2], o[1][3]), false, false);
+                        const int nb = nq + 8 * khalf;
+                        if (row_ok[fm] && nb + 7 < p.N)
+                            *reinterpret_cast<u32x4*>(orow[fm] + nb) = u32x4{s0[0], s1[0], s0[1], s1[1]};
+                    } else if (row_ok[fm]) {
+#pragma unroll
+                        for (int q = 0; q < 2; ++q)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const int n = nq + 8 * q + 4 * khalf + j;
+                                if (n < p.N) orow[fm][n] = (uint16_t)f32_to_bf16_bits(o[q][j]);
+                            }
+                    }
                 }
             }
         }
-    }
+    };
+    if (p.bias || p.bias2) run(std::true_type{});
+    else run(std::false_type{});
 }
 
 // fp32 operands: fp32 bias and output, no intermediate rounding, exact SiLU.
