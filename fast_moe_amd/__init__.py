@@ -2,6 +2,7 @@
 gfx950 (MI355X) HIP kernels behind the reference's operator API."""
 from .kernels.utils import KernelType
 from .modules.fast_moe_module import FastMoELayer, GatingNetwork
+from .modules.sgmoe import MRNOutput, SGConfig, SGMoE
 
 __version__ = "0.1.0"
-__all__ = ["FastMoELayer", "GatingNetwork", "KernelType", "__version__"]
+__all__ = ["FastMoELayer", "GatingNetwork", "KernelType", "MRNOutput", "SGConfig", "SGMoE", "__version__"]

@@ -88,6 +88,25 @@ __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores,
         const int e = v * LPT + sub;
         my[v] = (live && e < E) ? load_score<T>(scores + t * E + e) : ninf;
     }
+    // modes 2 and 3: the inputs are logits; they are L2-normalised over the experts first
+    // (F.normalize: l / max(||l||, 1e-12), rounded to the logits' dtype), and it is the
+    // normalised values that are ranked: rounding can tie values that differed before
+    if (renorm >= 2) {
+        float sq = 0.0f;
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            const int e = v * LPT + sub;
+            if (live && e < E) sq += my[v] * my[v];
+        }
+#pragma unroll
+        for (int o = LPT / 2; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+        const float norm = fmaxf(round_to<T>(sqrtf(sq)), 1e-12f);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            const int e = v * LPT + sub;
+            if (live && e < E) my[v] = round_to<T>(my[v] / norm);
+        }
+    }
     int rank[VPL];
 #pragma unroll
     for (int v = 0; v < VPL; ++v) rank[v] = 0;
@@ -112,13 +131,35 @@ __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores,
         const int e = v * LPT + sub;
         if (live && e < E && rank[v] < K) s_sel[wave][grp][rank[v]] = my[v];
     }
+    // gates of modes 2 and 3: softmax of the normalised logits over all experts (2) or over
+    // the K selected ones (3)
+    float soft_sum = 0.0f;
     __syncthreads();
+    if (renorm == 2) {
+        // the largest normalised logit is slot 0; exp(n_i - n_max) summed over all experts
+        const float nmax = live ? s_sel[wave][grp][0] : 0.0f;
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            const int e = v * LPT + sub;
+            if (live && e < E) soft_sum += expf(my[v] - nmax);
+        }
+#pragma unroll
+        for (int o = LPT / 2; o >= 1; o >>= 1) soft_sum += __shfl_xor(soft_sum, o, kWave);
+    }
     if (!live) return;
     float denom = 1.0f;
-    if (renorm) {
+    if (renorm == 1) {
         float s = 0.0f;
         for (int j = 0; j < K; ++j) s = s + fabsf(s_sel[wave][grp][j]);   // slot order
         denom = fmaxf(round_to<T>(s), round_to<T>(1e-12f));
+    }
+    float nmax = 0.0f;
+    if (renorm >= 2) {
+        nmax = s_sel[wave][grp][0];
+        if (renorm == 3) {
+            soft_sum = 0.0f;
+            for (int j = 0; j < K; ++j) soft_sum += expf(s_sel[wave][grp][j] - nmax);
+        }
     }
 #pragma unroll
     for (int v = 0; v < VPL; ++v) {
@@ -127,7 +168,10 @@ __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores,
             const int64_t p = t * K + rank[v];
             topk_idx[p] = e;
             compact[p] = (uint16_t)e;
-            store_score<T>(gates + p, renorm ? round_to<T>(my[v] / denom) : my[v]);
+            float g = my[v];
+            if (renorm == 1) g = round_to<T>(my[v] / denom);
+            else if (renorm >= 2) g = round_to<T>(expf(my[v] - nmax) / soft_sum);
+            store_score<T>(gates + p, g);
         }
     }
 }
@@ -340,6 +384,7 @@ extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, i
     hipStream_t stream = (hipStream_t)stream_;
     if (int rc = check_common(T, E, K, workspace, workspace_bytes, "fmoe_route_topk")) return rc;
     FMOE_REQUIRE(K <= E, "fmoe_route_topk: K=%d > E=%d", K, E);
+    FMOE_REQUIRE(renorm >= 0 && renorm <= 3, "fmoe_route_topk: gate mode %d is not one of 0..3", renorm);
     FMOE_REQUIRE(score_dtype == FMOE_F32 || score_dtype == FMOE_BF16,
                  "fmoe_route_topk: scores must be fp32 or bf16");
     FMOE_REQUIRE(lengths && offsets, "fmoe_route_topk: lengths/offsets are NULL");

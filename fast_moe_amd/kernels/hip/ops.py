@@ -57,8 +57,12 @@ def _rows_contiguous(t: torch.Tensor) -> torch.Tensor:
 
 
 # ------------------------------------------------------------------- routing
-def route_topk(scores: torch.Tensor, k: int, renorm: bool = True) -> Dict[str, torch.Tensor]:
-    """scores [T, E] (fp32 / bf16 gate probabilities) -> routing tensors, see fmoe_route_topk."""
+GATE_RAW, GATE_L1, GATE_SOFTMAX_ALL, GATE_SOFTMAX_TOPK = 0, 1, 2, 3
+
+
+def route_topk(scores: torch.Tensor, k: int, renorm=True) -> Dict[str, torch.Tensor]:
+    """scores [T, E] (fp32 / bf16 gate probabilities, or router logits for the softmax modes)
+    -> routing tensors, see fmoe_route_topk.  ``renorm``: bool, or one of the GATE_* modes."""
     dev = _need_cuda("route_topk", scores)
     if scores.ndim != 2:
         raise ValueError("route_topk: scores must be [T, E]")

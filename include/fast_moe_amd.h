@@ -66,8 +66,12 @@ size_t fmoe_route_workspace_bytes(int64_t T, int E, int K);
  * torch.ops.fbgemm.asynchronous_complete_cumsum call at :131.
  *
  *   scores        [T, E] row-major, FMOE_F32 or FMOE_BF16 (softmax output)
- *   renorm        1: gates = v / max(sum|v|, 1e-12) in the scores' dtype
- *                 (F.normalize, :103); 0: gates = selected scores
+ *   renorm        gate mode.  0: gates = selected scores.
+ *                 1: gates = v / max(sum|v|, 1e-12) in the scores' dtype (F.normalize, :103).
+ *                 2, 3: `scores` are router LOGITS, the SGMoE router of utils/utils.py:139-164
+ *                 (_compute_top_logits): logits L2-normalised over the experts, selection in
+ *                 descending stable order, gates = softmax of the normalised logits over all
+ *                 experts (2, post_softmax=False) or over the K selected ones (3, post_softmax=True)
  * outputs
  *   topk_idx      [T, K] int64  selected experts; slot order = descending score,
  *                               equal scores -> lower expert id first
