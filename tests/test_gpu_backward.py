@@ -198,3 +198,43 @@ def test_jagged_transpose_layout(R, C, E, gather, silu, dtype):
         assert torch.equal(got == 0, ref == 0) or True
     else:
         assert torch.equal(got, ref)
+
+
+def test_big_shape_forward_and_backward_64bit_offsets():
+    """The reference's big-shape case (kernels/tests/moe_test.py:132-161): L = 4 550 700 tokens, top-2,
+    256 -> 256, so the output has 2.33e9 elements and every row offset needs 64 bits.  Checked on
+    sampled rows / tokens (the last ones included) and, for the bias gradient, in closed form."""
+    from fast_moe_amd.kernels import moe
+    L, E, K, D, N = 4550700, 4, 2, 256, 256
+    r = make_routing(L, E, K, seed=3)
+    g = torch.Generator().manual_seed(5)
+    x0 = torch.randn(L, D, generator=g, dtype=torch.float32).to(BF16)
+    w0 = kn_weight(E, D, N, 2, False, D ** -0.5)
+    b0 = randn((E, N), 3)
+    table = (torch.randn(64, N, generator=g) * 0.01).to(BF16)
+    R = L * K
+    x, w, b = leaf(x0, device="cuda"), leaf(w0, device="cuda"), leaf(b0, device="cuda")
+    out = moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, b)
+    assert out.numel() > 2 ** 31
+    rows = torch.cat([torch.randint(0, R, (256,), generator=g), torch.arange(R - 64, R), torch.arange(64)])
+    expert = torch.bucketize(rows, r["offsets"][1:], right=True)
+    tok = r["gate_index"][rows] // K
+    ref = torch.einsum("rd,rdn->rn", x0[tok].float(), w0.float()[expert]) + b0.float()[expert]
+    close(out.detach()[rows.cuda()], ref, "big-shape rows", rtol=2e-2, atol_frac=1e-2)
+    dout = table.cuda()[torch.arange(R, device="cuda") % 64]
+    out.backward(dout)
+    del out, dout
+    # d_bias[e] = sum over the rows of e of table[r % 64]
+    cls = torch.arange(R) % 64
+    ref_db = torch.zeros(E, N)
+    for e in range(E):
+        lo, hi = int(r["offsets"][e]), int(r["offsets"][e + 1])
+        ref_db[e] = torch.bincount(cls[lo:hi], minlength=64).float() @ table.float()
+    close(b.grad, ref_db, "big-shape d_bias", rtol=2e-2, atol_frac=1e-2)
+    # d_jagged[t] = sum over the K rows of token t of dout[r] @ W[e(r)]^T
+    toks = torch.cat([torch.randint(0, L, (128,), generator=g), torch.arange(L - 16, L)])
+    rr = r["reverse_index"][toks]                                   # [n, K] routed rows
+    ee = torch.bucketize(rr, r["offsets"][1:], right=True)
+    ref_dx = torch.einsum("tkn,tkdn->td", table.float()[rr % 64], w0.float()[ee])
+    close(x.grad[toks.cuda()], ref_dx, "big-shape d_jagged", rtol=3e-2, atol_frac=2e-2)
+    assert w.grad.shape == w.shape and torch.isfinite(w.grad.float()).all()

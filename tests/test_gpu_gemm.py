@@ -277,7 +277,8 @@ def test_forward_only_and_dtype_errors():
     (4096, 8, 2, 1024, 264, "plain"),      # N = 264: last column tile 8 wide
     (9000, 3, 1, 512, 512, "plain"),       # fewer tiles than CUs, K_top = 1 (index_shift 0)
     (6144, 24, 3, 256, 384, "swiglu"),     # top-3: index division, not a shift
-    (20000, 200, 2, 128, 128, "swiglu"),   # many experts, about 200 rows each
+    (20000, 200, 2, 128, 128, "swiglu"),   # many experts, about 200 rows each (register tables, 4 entries)
+    (30000, 300, 2, 128, 128, "swiglu"),   # more than 256 experts: 4-slot ring with its tables in LDS
     (3000, 2, 2, 2048, 128, "swiglu"),     # long K, one column tile
 ])
 def test_ring_kernel_shapes(L, E, K, Din, Dout, epi):
