@@ -53,6 +53,12 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     const bool f32 = d->a_dtype == FMOE_F32;
     const bool swiglu = d->epilogue == FMOE_EPI_SWIGLU;
     if (swiglu) FMOE_REQUIRE(d->b2 != nullptr, "fmoe_grouped_gemm: SWIGLU needs b2");
+    FMOE_REQUIRE((d->aux == nullptr) == (d->aux2 == nullptr), "fmoe_grouped_gemm: aux and aux2 come together");
+    if (d->aux) {
+        FMOE_REQUIRE(swiglu, "fmoe_grouped_gemm: aux outputs are the SWIGLU pre-activations");
+        FMOE_REQUIRE(d->aux_stride_row >= d->n, "fmoe_grouped_gemm: aux row stride %lld < n %d",
+                     (long long)d->aux_stride_row, d->n);
+    }
     if (fp8) {
         FMOE_REQUIRE(d->a_scale && d->b_scale, "fmoe_grouped_gemm: e4m3 operands need a_scale and b_scale");
         if (swiglu) FMOE_REQUIRE(d->b2_scale != nullptr, "fmoe_grouped_gemm: SWIGLU e4m3 needs b2_scale");
@@ -91,7 +97,12 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     // 16-byte stores: 8 bf16 (4 fp32) output columns at a time
     const int vec_cols = f32 ? 4 : 8;
     p.k_window = d->k_window;
-    p.vec_store = (d->n % vec_cols == 0) && (d->out_stride_row % vec_cols == 0) && aligned16(d->out);
+    p.k_window_multiple = d->k_window ? d->k_window_multiple : 0;
+    p.aux = (uint16_t*)d->aux;
+    p.aux2 = (uint16_t*)d->aux2;
+    p.aux_stride = d->aux_stride_row;
+    p.vec_store = (d->n % vec_cols == 0) && (d->out_stride_row % vec_cols == 0) && aligned16(d->out) &&
+                  (!d->aux || ((d->aux_stride_row % vec_cols == 0) && aligned16(d->aux) && aligned16(d->aux2)));
 
     const int esize = fp8 ? 1 : (f32 ? 4 : 2);
     const int chunk = 16 / esize;

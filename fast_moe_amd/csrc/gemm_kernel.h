@@ -65,6 +65,10 @@ struct GemmParams {
     int n_tiles;
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
     const int64_t* k_window;            // [E+1] per-expert contraction range, or null
+    int k_window_multiple;              // every window is a multiple of this and at least twice it (0: unknown)
+    uint16_t* aux;                      // SWIGLU: the two pre-activations, or null
+    uint16_t* aux2;
+    int64_t aux_stride;
 };
 
 constexpr int kDtBf16 = 0, kDtE4m3 = 1, kDtF32 = 2;
@@ -136,8 +140,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         if (FP8) rsa[fm] = 1.0f / p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))];
     }
     // the bias-free form (FastMoE's SwiGLU experts, every fp8 call without bias) skips the adds
-    auto run = [&](auto has_bias_c) {
+    auto run = [&](auto has_bias_c, auto has_aux_c) {
         constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
+        constexpr bool HAS_AUX = SWIGLU && decltype(has_aux_c)::value;   // keep the pre-activations (training)
         // per-column epilogue constants of this lane: [fn][gp][q][j] <-> column nq + 8*q + 4*khalf + j
         // with nq = first column of register-quad pair gp of fragment fn
         float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
@@ -165,7 +170,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 #pragma unroll
                 for (int gp = 0; gp < 2; ++gp) {
                     const int nq = col0 + fn * 32 + 16 * gp;
-                    float o[2][4];
+                    float o[2][4], pg[2][4], pu[2][4];
 #pragma unroll
                     for (int q = 0; q < 2; ++q)
 #pragma unroll
@@ -184,35 +189,50 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                 y = rbf(HAS_BIAS ? y + bv[fn][gp][q][j] : y);
                                 if (SWIGLU) y2 = rbf(HAS_BIAS ? y2 + bv2[fn][gp][q][j] : y2);
                             }
+                            pg[q][j] = y;
+                            pu[q][j] = y2;
                             if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
                             if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
                             o[q][j] = y;
                         }
-                    if (p.vec_store) {
-                        // pair the quads of the two lane halves: low lanes end up with columns
-                        // nq..nq+7, high lanes with nq+8..nq+15 of their row
-                        const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][0], o[0][1]),
-                                                                          pack_bf16(o[1][0], o[1][1]), false, false);
-                        const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pack_bf16(o[0][2], o[0][3]),
-                                                                          pack_bf16(o[1][2], o[1][3]), false, false);
-                        const int nb = nq + 8 * khalf;
-                        if (row_ok[fm] && nb + 7 < p.N)
-                            *reinterpret_cast<u32x4*>(orow[fm] + nb) = u32x4{s0[0], s1[0], s0[1], s1[1]};
-                    } else if (row_ok[fm]) {
+                    auto store = [&](const float (&val)[2][4], uint16_t* dst) {
+                        if (p.vec_store) {
+                            // pair the quads of the two lane halves: low lanes end up with columns
+                            // nq..nq+7, high lanes with nq+8..nq+15 of their row
+                            const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(val[0][0], val[0][1]),
+                                                                              pack_bf16(val[1][0], val[1][1]), false, false);
+                            const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pack_bf16(val[0][2], val[0][3]),
+                                                                              pack_bf16(val[1][2], val[1][3]), false, false);
+                            const int nb = nq + 8 * khalf;
+                            if (row_ok[fm] && nb + 7 < p.N)
+                                *reinterpret_cast<u32x4*>(dst + nb) = u32x4{s0[0], s1[0], s0[1], s1[1]};
+                        } else if (row_ok[fm]) {
 #pragma unroll
-                        for (int q = 0; q < 2; ++q)
+                            for (int q = 0; q < 2; ++q)
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                const int n = nq + 8 * q + 4 * khalf + j;
-                                if (n < p.N) orow[fm][n] = (uint16_t)f32_to_bf16_bits(o[q][j]);
-                            }
+                                for (int j = 0; j < 4; ++j) {
+                                    const int n = nq + 8 * q + 4 * khalf + j;
+                                    if (n < p.N) dst[n] = (uint16_t)f32_to_bf16_bits(val[q][j]);
+                                }
+                        }
+                    };
+                    store(o, orow[fm]);
+                    if (HAS_AUX) {
+                        const int64_t aux_off = (row0 + wm * TM + fm * 32 + (lane & 31)) * p.aux_stride;
+                        store(pg, p.aux + aux_off);
+                        store(pu, p.aux2 + aux_off);
                     }
                 }
             }
         }
     };
-    if (p.bias || p.bias2) run(std::true_type{});
-    else run(std::false_type{});
+    if (SWIGLU && p.aux) {
+        if (p.bias || p.bias2) run(std::true_type{}, std::true_type{});
+        else run(std::false_type{}, std::true_type{});
+    } else {
+        if (p.bias || p.bias2) run(std::true_type{}, std::false_type{});
+        else run(std::false_type{}, std::false_type{});
+    }
 }
 
 // fp32 operands: fp32 bias and output, no intermediate rounding, exact SiLU.
@@ -244,20 +264,29 @@ __device__ __forceinline__ void gemm_epilogue_f32(const GemmParams& p, f32x16 (&
                 const int tile_row = wm * TM + fm * 32 + (lane & 31);
                 if (tile_row >= rows_valid) continue;
                 float* orow = out + (row0 + tile_row) * p.out_stride;
-                float o[4];
+                float o[4], pg[4], pu[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     float y = acc[fn][fm][4 * g + j] + bv[j];
+                    pg[j] = y;
+                    pu[j] = SWIGLU ? acc[fn + FN / 2][fm][4 * g + j] + bv2[j] : 0.0f;
                     if (EPI == FMOE_EPI_SILU) y = silu_f32(y);
-                    if (SWIGLU) y = silu_f32(y) * (acc[fn + FN / 2][fm][4 * g + j] + bv2[j]);
+                    if (SWIGLU) y = silu_f32(y) * pu[j];
                     o[j] = y;
                 }
-                if (p.vec_store && nb + 3 < p.N) {
-                    *reinterpret_cast<f32x4*>(orow + nb) = f32x4{o[0], o[1], o[2], o[3]};
-                } else {
+                auto store = [&](const float (&val)[4], float* dst) {
+                    if (p.vec_store && nb + 3 < p.N) {
+                        *reinterpret_cast<f32x4*>(dst + nb) = f32x4{val[0], val[1], val[2], val[3]};
+                    } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (nb + j < p.N) orow[nb + j] = o[j];
+                        for (int j = 0; j < 4; ++j)
+                            if (nb + j < p.N) dst[nb + j] = val[j];
+                    }
+                };
+                store(o, orow);
+                if (SWIGLU && p.aux) {
+                    store(pg, reinterpret_cast<float*>(p.aux) + (row0 + tile_row) * p.aux_stride);
+                    store(pu, reinterpret_cast<float*>(p.aux2) + (row0 + tile_row) * p.aux_stride);
                 }
             }
         }

@@ -93,24 +93,27 @@ class IndexSelectJaggedBmm(torch.autograd.Function):
     @staticmethod
     def forward(ctx, offsets, index, jagged, weight, bias, weight_p, bias_p):
         swiglu = weight_p is not None
+        pre = None
+        if swiglu:   # both pre-activations are kept for the backward pass, as the reference does
+            out_dtype = torch.float32 if jagged.dtype == torch.float32 else torch.bfloat16
+            pre = tuple(torch.empty((index.numel(), weight.shape[2]), dtype=out_dtype, device=jagged.device)
+                        for _ in range(2))
         out = ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                                index_div=index.shape[-1], bias=bias, b2=weight_p, bias2=bias_p,
-                               epilogue=EPI_SWIGLU if swiglu else EPI_NONE)
-        ctx.save_for_backward(offsets, index, jagged, weight, bias, weight_p, bias_p)
+                               epilogue=EPI_SWIGLU if swiglu else EPI_NONE, aux=pre)
+        ctx.save_for_backward(offsets, index, jagged, weight, bias, weight_p, bias_p, *(pre or (None, None)))
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        offsets, index, jagged, weight, bias, weight_p, bias_p = ctx.saved_tensors
+        offsets, index, jagged, weight, bias, weight_p, bias_p, g, u = ctx.saved_tensors
         K = index.shape[-1]
         R = index.numel()
         dout = dout.contiguous()
         swiglu = weight_p is not None
-        if swiglu:   # the pre-activations are recomputed, not kept from the forward
-            gemm = lambda w, b: ops.grouped_gemm(offsets, jagged, w, total_rows=R, row_index=index,
-                                                 index_div=K, bias=b)
-            g, u = gemm(weight, bias), gemm(weight_p, bias_p)
+        if swiglu:
             dg, du = ops.swiglu_bwd(g, u, dout)
+            del g, u
             drows, weights = [dg, du], [weight, weight_p]
         else:
             drows, weights = [dout], [weight]

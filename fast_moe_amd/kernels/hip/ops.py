@@ -185,10 +185,13 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  bias2: Optional[torch.Tensor] = None, epilogue: int = EPI_NONE, a_silu: bool = False,
                  a_scale: Optional[torch.Tensor] = None, b_scale: Optional[torch.Tensor] = None,
                  b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0,
-                 k_window: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 k_window: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                 k_window_multiple: int = 0,
+                 aux: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
     strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
-    [total_rows, N] in bf16 (fp32 for fp32 operands)."""
+    [total_rows, N] in bf16 (fp32 for fp32 operands).  ``aux`` = two tensors like the output
+    that receive the SWIGLU pre-activations."""
     dev = _need_cuda("grouped_gemm", offsets, a, b, row_index, bias, b2, bias2, a_scale, b_scale, b2_scale)
     fp8 = a.dtype == FP8_DTYPE
     if not fp8 and a.dtype not in (torch.bfloat16, torch.float32):
@@ -229,6 +232,14 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     elif (tuple(out.shape) != (total_rows, N) or out.dtype != out_dtype or out.device != dev
           or out.stride(1) != 1):
         raise ValueError(f"grouped_gemm: out must be {out_dtype} [{total_rows}, {N}] with contiguous rows")
+    if aux is not None:
+        if epilogue != EPI_SWIGLU:
+            raise ValueError("grouped_gemm: aux outputs exist for the SWIGLU epilogue only")
+        for t in aux:
+            if (tuple(t.shape) != (total_rows, N) or t.dtype != out_dtype or t.device != dev or t.stride(1) != 1
+                    or t.stride(0) != aux[0].stride(0)):
+                raise ValueError(f"grouped_gemm: aux tensors must be {out_dtype} [{total_rows}, {N}] with "
+                                 "contiguous rows and one row stride")
     if total_rows == 0:
         return out
 
@@ -278,6 +289,9 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.out = out.data_ptr()
     d.out_stride_row = out.stride(0)
     d.k_window = _ptr(k_window)
+    d.k_window_multiple = k_window_multiple if k_window is not None else 0
+    if aux is not None:
+        d.aux, d.aux2, d.aux_stride_row = aux[0].data_ptr(), aux[1].data_ptr(), aux[0].stride(0)
     rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
     _lib.check(rc, "fmoe_grouped_gemm")
     return out

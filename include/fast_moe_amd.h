@@ -192,6 +192,15 @@ typedef struct fmoe_gemm_desc {
     const int64_t* k_window; /* NULL, or [E+1]: expert e contracts over the k range
                                 [k_window[e], k_window[e+1]) of A and B (then `k` is
                                 only an upper bound); values multiples of 8          */
+    int32_t k_window_multiple; /* 0, or a promise of the caller: every window length is a
+                                multiple of this many elements and at least twice it
+                                (64 or more lets the LDS-ring kernel take the call)   */
+    int32_t reserved0;      /* 0                                                  */
+    void* aux;              /* NULL, or with FMOE_EPI_SWIGLU [total_rows, n] in out_dtype:  */
+    void* aux2;             /* receive A x B + bias (aux) and A x B2 + bias2 (aux2), the
+                                two pre-activations the backward pass needs (the ALPHA and
+                                BETA outputs of kernels/triton/triton_moe.py:2316-2345) */
+    int64_t aux_stride_row;
 } fmoe_gemm_desc;
 
 int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);

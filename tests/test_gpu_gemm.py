@@ -461,3 +461,42 @@ def test_fp32_swiglu_gating_3d_and_combine():
         out = moe.silu_jagged_bmm_combine(0, dev(r["offsets"]), dev(jag), dev(w), dev(b), dev(r["token_index"]),
                                           dev(r["reverse_index"]), dev(gates), dev(r["gate_index"]), has_silu=True)
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,dtype,bias", [
+    (4096, 8, 2, 256, 384, "bf16", True),     # ring kernel
+    (4096, 8, 2, 256, 384, "bf16", False),
+    (300, 4, 2, 72, 40, "bf16", True),        # element kernel, scalar stores
+    (1000, 4, 2, 64, 128, "f32", True),
+    (4096, 8, 2, 256, 384, "fp8", True),
+])
+def test_swiglu_pre_activation_outputs(L, E, K, Din, Dout, dtype, bias):
+    """aux / aux2 of the SWIGLU epilogue are bit for bit the outputs of the two plain GEMMs, and the
+    main output does not change when they are requested."""
+    from fast_moe_amd.kernels.hip import ops
+    from fast_moe_amd.kernels.hip._lib import EPI_SWIGLU
+    r = make_routing(L, E, K, seed=L)
+    td = torch.float32 if dtype == "f32" else BF16
+    x = randn((L, Din), 1).to(td).cuda()
+    w = weights(E, Din, Dout, 2, False, Din ** -0.5).to(td).cuda()
+    wp = weights(E, Din, Dout, 3, False, Din ** -0.5).to(td).cuda()
+    b = randn((E, Dout), 4).to(td).cuda() if bias else None
+    bp = randn((E, Dout), 5).to(td).cuda() if bias else None
+    kw = dict(total_rows=L * K, row_index=dev(r["index"]), index_div=K)
+    sc = [{}, {}, {}]
+    if dtype == "fp8":
+        xq, xs = ops.quant_rows_fp8(x)
+        wq, ws = ops.quant_rows_fp8(w.permute(0, 2, 1))
+        wpq, wps = ops.quant_rows_fp8(wp.permute(0, 2, 1))
+        x, w, wp = xq, wq.permute(0, 2, 1), wpq.permute(0, 2, 1)
+        sc = [dict(a_scale=xs, b_scale=ws), dict(a_scale=xs, b_scale=wps), dict(a_scale=xs, b_scale=ws, b2_scale=wps)]
+    off = dev(r["offsets"])
+    g = ops.grouped_gemm(off, x, w, bias=b, **kw, **sc[0])
+    u = ops.grouped_gemm(off, x, wp, bias=bp, **kw, **sc[1])
+    plain = ops.grouped_gemm(off, x, w, bias=b, b2=wp, bias2=bp, epilogue=EPI_SWIGLU, **kw, **sc[2])
+    aux = (torch.full_like(g, 7.0), torch.full_like(g, 7.0))
+    out = ops.grouped_gemm(off, x, w, bias=b, b2=wp, bias2=bp, epilogue=EPI_SWIGLU, aux=aux, **kw, **sc[2])
+    assert torch.equal(out, plain)
+    assert torch.equal(aux[0], g) and torch.equal(aux[1], u)
+    with pytest.raises(ValueError, match="SWIGLU"):
+        ops.grouped_gemm(off, x, w, bias=b, aux=aux, **kw, **sc[0])
