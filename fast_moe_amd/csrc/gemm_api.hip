@@ -29,8 +29,9 @@ int lds_per_block() {
 }
 }  // namespace fmoe
 
-extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
+// Checks the descriptor, fills the kernel parameters and picks the kernel.  sel < 0: nothing to do.
+static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
+    sel = -1;
     FMOE_REQUIRE(d != nullptr, "fmoe_grouped_gemm: desc is NULL");
     FMOE_REQUIRE(d->num_experts >= 1 && d->n >= 1 && d->k >= 1,
                  "fmoe_grouped_gemm: need E, n, k >= 1 (E=%d n=%d k=%d)", d->num_experts, d->n, d->k);
@@ -41,7 +42,7 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
                  "fmoe_grouped_gemm: output must be bf16 (fp32 for fp32 operands)");
     FMOE_REQUIRE(d->epilogue >= FMOE_EPI_NONE && d->epilogue <= FMOE_EPI_SWIGLU,
                  "fmoe_grouped_gemm: unknown epilogue %d", d->epilogue);
-    if (d->total_rows == 0) return FMOE_OK;
+    if (d->total_rows == 0) return FMOE_OK;     // sel stays -1
     FMOE_REQUIRE(d->offsets && d->a && d->b && d->out, "fmoe_grouped_gemm: NULL tensor pointer");
     FMOE_REQUIRE(d->a_rows >= 1, "fmoe_grouped_gemm: a_rows < 1");
     FMOE_REQUIRE(d->index_div >= 1, "fmoe_grouped_gemm: index_div < 1");
@@ -65,7 +66,6 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
         FMOE_REQUIRE(!d->a_silu, "fmoe_grouped_gemm: a_silu is not defined for e4m3 operands");
     }
 
-    GemmParams p;
     p.offsets = d->offsets;
     p.row_index = d->row_index;
     p.E = d->num_experts;
@@ -101,8 +101,12 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     p.aux = (uint16_t*)d->aux;
     p.aux2 = (uint16_t*)d->aux2;
     p.aux_stride = d->aux_stride_row;
+    // (the vector-store path addresses a row inside a 32-row block with a 32-bit byte offset)
+    const int64_t stride_cap = (int64_t)1 << 25;
     p.vec_store = (d->n % vec_cols == 0) && (d->out_stride_row % vec_cols == 0) && aligned16(d->out) &&
-                  (!d->aux || ((d->aux_stride_row % vec_cols == 0) && aligned16(d->aux) && aligned16(d->aux2)));
+                  d->out_stride_row < stride_cap &&
+                  (!d->aux || ((d->aux_stride_row % vec_cols == 0) && aligned16(d->aux) && aligned16(d->aux2) &&
+                               d->aux_stride_row < stride_cap));
 
     const int esize = fp8 ? 1 : (f32 ? 4 : 2);
     const int chunk = 16 / esize;
@@ -119,10 +123,37 @@ extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_)
     const int64_t span32 = ((int64_t)1 << 32) - 4096;
     const bool near = d->a_rows * d->a_stride_row * esize + (int64_t)d->k * esize < span32 &&
                       (int64_t)d->n * d->b_stride_n * esize + (int64_t)d->k * esize < span32;
-    const bool ring = fast && big && !f32 && !d->a_silu && !d->k_window && (d->k % slice) == 0 && d->k / slice >= 3 &&
+    const bool ring = fast && big && !f32 && !d->a_silu && (d->k % slice) == 0 && d->k / slice >= 3 &&
                       p.vec_store && d->num_experts <= 1024 && d->total_rows < ((int64_t)1 << 31) * 128 && near;
-    const int sel = !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
-    if (fp8) return run_gemm_fp8(p, d->epilogue, sel, stream);
-    if (f32) return run_gemm_f32(p, d->epilogue, d->a_silu != 0, sel, stream);
+    // N-contiguous bf16 weights (B[e][k][n], n fastest) are read in place by the paired ring
+    const bool ring_tr = !fp8 && !f32 && big && !d->a_silu && !d->k_window && d->b_stride_n == 1 &&
+                         d->b_stride_k != 1 && (d->b_stride_k % chunk) == 0 && (d->b_stride_e % chunk) == 0 &&
+                         (d->a_stride_row % chunk) == 0 && (d->a_stride_e % chunk) == 0 && aligned16(d->a) &&
+                         aligned16(d->b) && (!swiglu || aligned16(d->b2)) && (d->k % (2 * slice)) == 0 &&
+                         d->k / slice >= 4 && p.vec_store && d->num_experts <= TileRing5W::kMaxExperts &&
+                         d->total_rows < ((int64_t)1 << 31) && lds_per_block() >= TileRing5::LDS_BYTES &&
+                         d->a_rows * d->a_stride_row * esize + (int64_t)d->k * esize < span32 &&
+                         ((int64_t)d->k * d->b_stride_k + d->n) * esize < span32;
+    sel = ring_tr ? kSelRing : !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_grouped_gemm(const fmoe_gemm_desc* d, fmoe_stream_t stream_) {
+    hipStream_t stream = (hipStream_t)stream_;
+    GemmParams p;
+    int sel;
+    if (int rc = prepare_gemm(d, p, sel)) return rc;
+    if (sel < 0) return FMOE_OK;
+    if (d->a_dtype == FMOE_E4M3) return run_gemm_fp8(p, d->epilogue, sel, stream);
+    if (d->a_dtype == FMOE_F32) return run_gemm_f32(p, d->epilogue, d->a_silu != 0, sel, stream);
     return run_gemm_bf16(p, d->epilogue, d->a_silu != 0, sel, stream);
+}
+
+extern "C" int fmoe_grouped_gemm_plan(const fmoe_gemm_desc* d, int* plan) {
+    FMOE_REQUIRE(plan != nullptr, "fmoe_grouped_gemm_plan: plan is NULL");
+    GemmParams p;
+    int sel;
+    if (int rc = prepare_gemm(d, p, sel)) return rc;
+    *plan = sel < 0 ? FMOE_PLAN_NONE : sel;
+    return FMOE_OK;
 }

@@ -114,6 +114,11 @@ __device__ __forceinline__ u32x4 silu_f32x4(u32x4 v) {
     return v;
 }
 
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
 // ------------------------------------------------------------------------ epilogue
 // acc[fn][fm][v]: fragment (fn, fm) of the wave tile, v = 4*g + j <-> output row
 // (lane & 31) of fragment row block fm, output column 32*fn + 8*g + 4*(lane >> 5) + j.
@@ -128,14 +133,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
     const int khalf = lane >> 5;
     const int64_t bias_row = (int64_t)expert * p.bias_se;
+    // Output addresses are a wave-uniform 64-bit base (tile row block, column group: scalar
+    // registers and scalar arithmetic) plus one 32-bit per-lane byte offset (the lane's row
+    // inside the 32-row block and its 16-byte half): no per-row pointers to keep in vector
+    // registers over an epilogue whose accumulators and column constants already fill them.
+    wm = __builtin_amdgcn_readfirstlane(wm);
+    wn = __builtin_amdgcn_readfirstlane(wn);
+    row0 = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) |
+                     (uint32_t)__builtin_amdgcn_readfirstlane((int)row0));
+    const uint32_t out_lane = (uint32_t)(lane & 31) * (uint32_t)p.out_stride * 2u + (uint32_t)khalf * 16u;
+    const uint32_t aux_lane = (uint32_t)(lane & 31) * (uint32_t)p.aux_stride * 2u + (uint32_t)khalf * 16u;
     float rsa[FM];
     bool row_ok[FM];
-    uint16_t* orow[FM];
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
         const int tile_row = wm * TM + fm * 32 + (lane & 31);
         row_ok[fm] = tile_row < rows_valid;
-        orow[fm] = p.out + (row0 + tile_row) * p.out_stride;
         rsa[fm] = 1.0f;
         if (FP8) rsa[fm] = 1.0f / p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))];
     }
@@ -195,7 +208,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                             if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
                             o[q][j] = y;
                         }
-                    auto store = [&](const float (&val)[2][4], uint16_t* dst) {
+                    // base: first element of the 32-row block's first row (wave-uniform)
+                    auto store = [&](const float (&val)[2][4], uint16_t* base, uint32_t lane_off, int64_t stride) {
                         if (p.vec_store) {
                             // pair the quads of the two lane halves: low lanes end up with columns
                             // nq..nq+7, high lanes with nq+8..nq+15 of their row
@@ -205,8 +219,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                                                               pack_bf16(val[1][2], val[1][3]), false, false);
                             const int nb = nq + 8 * khalf;
                             if (row_ok[fm] && nb + 7 < p.N)
-                                *reinterpret_cast<u32x4*>(dst + nb) = u32x4{s0[0], s1[0], s0[1], s1[1]};
+                                *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(base + nq) + lane_off) =
+                                    u32x4{s0[0], s1[0], s0[1], s1[1]};
                         } else if (row_ok[fm]) {
+                            uint16_t* dst = base + (int64_t)(lane & 31) * stride;
 #pragma unroll
                             for (int q = 0; q < 2; ++q)
 #pragma unroll
@@ -216,15 +232,22 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                 }
                         }
                     };
-                    store(o, orow[fm]);
+                    const int64_t block_row = row0 + wm * TM + fm * 32;
+                    store(o, p.out + block_row * p.out_stride, out_lane, p.out_stride);
                     if (HAS_AUX) {
-                        const int64_t aux_off = (row0 + wm * TM + fm * 32 + (lane & 31)) * p.aux_stride;
-                        store(pg, p.aux + aux_off);
-                        store(pu, p.aux2 + aux_off);
+                        store(pg, p.aux + block_row * p.aux_stride, aux_lane, p.aux_stride);
+                        store(pu, p.aux2 + block_row * p.aux_stride, aux_lane, p.aux_stride);
                     }
                 }
             }
         }
+        // Everything older than this epilogue's own stores has completed: a wait that costs
+        // nothing (the loads it names were needed above) but tells the compiler so.  Without it
+        // a spill reload that one of the branches above leaves unused stays "pending" in the
+        // compiler's count, and the wait for it lands where its register is next written:
+        // inside the caller's steady-state loop, where it would also drain the LDS-DMA stream,
+        // which the compiler cannot see, on every iteration.
+        wait_vmcnt<FM * FN_OUT * 2 * (HAS_AUX ? 3 : 1)>();      // (the scalar-store path issues more)
     };
     if (SWIGLU && p.aux) {
         if (p.bias || p.bias2) run(std::true_type{}, std::true_type{});
@@ -667,17 +690,28 @@ __device__ __forceinline__ void dma16(const uint8_t* base, uint32_t voff, uint32
                  :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");
 }
 
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
-    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-
 __device__ __forceinline__ int uniform_lane(int v, int src_lane) {
     return __builtin_amdgcn_readfirstlane(wave_bcast(v, src_lane));
 }
 
-template <typename TL, bool FP8, int EPI>
+//
+// WTR: the weights are N-contiguous (B[e][k][n] with b_sn == 1, an [E, K, N]-contiguous tensor or
+// the transposed view the input-gradient GEMM multiplies by) and are consumed in place.  A ring
+// slot then holds the weight part of a K-slice as two blocks [32 k][128 n] of 256-byte rows (n
+// 0..127 and 128..255 of the tile; gate and up columns with SWIGLU); LDS position p of row k
+// holds 16-byte chunk p ^ 4*(k%4) of that row, and the fragments are read with
+// ds_read_b64_tr_b16: within 16 lanes, lane j receives column j of 4 consecutive rows when lane
+// i points at row i/4, columns 4*(i%4)..+3, so two reads give a lane its 8 k values of one
+// column.  The four rows of a read and the two 16-lane groups served together fall into eight
+// different 32-byte bank groups.  bf16, paired ring only.
+//
+// KWIN: every expert contracts over its own window of K (p.k_window): the weight-gradient
+// GEMM.  Paired ring only; windows are whole pairs of K-slices, at least two pairs.
+template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false>
 __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmParams p) {
+    static_assert(!WTR || (TL::PAIR && !FP8 && TL::BN == 256 && TL::NW == 8),
+                  "in-place N-contiguous weights: bf16, paired ring, 256-column tiles of 8 waves");
+    static_assert(!KWIN || (TL::PAIR && !WTR), "contraction windows: paired ring, K-contiguous weights");
     constexpr int BM = TL::BM, BN = TL::BN, NW = TL::NW, STAGES = TL::STAGES;
     constexpr int FM = TL::FM, FN = TL::FN, TM = TL::TM, TN = TL::TN;
     constexpr bool PAIR = TL::PAIR;
@@ -746,17 +780,36 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         total_m = s_tab[p.E];
         r_first[0] = r_lo[0] = r_len[0] = 0;
     }
+    // The tiles of an XCD, numbered 0 .. xcd_count-1.  Without a contraction window: one
+    // contiguous range of the tile order (neighbouring tiles share operands in the XCD's L2).
+    // With one the cost of a tile follows its expert's row count, so whole groups go round
+    // robin over the XCDs instead (a contiguous range would hand one XCD all the long experts).
     const int64_t total_tiles = (int64_t)total_m * p.n_tiles;
     const int nslots = gridDim.x / kNumXcd;
-    const int64_t per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
-    const int64_t xcd_begin = xcd * per_xcd;
-    int64_t xcd_end = xcd_begin + per_xcd;
-    if (xcd_end > total_tiles) xcd_end = total_tiles;
+    const int64_t group_span = (int64_t)kGroupM * p.n_tiles;
+    constexpr bool windowed = KWIN;
+    int64_t xcd_begin, xcd_count;
+    if (windowed) {
+        const int64_t n_groups = (total_m + kGroupM - 1) / kGroupM;
+        const int64_t mine = n_groups > xcd ? (n_groups - xcd + kNumXcd - 1) / kNumXcd : 0;
+        xcd_begin = 0;
+        xcd_count = mine * group_span;
+        if (mine > 0 && (n_groups - 1) % kNumXcd == xcd)   // the last group may be short
+            xcd_count -= n_groups * group_span - total_tiles;
+    } else {
+        const int64_t per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
+        xcd_begin = xcd * per_xcd;
+        xcd_count = total_tiles - xcd_begin < per_xcd ? total_tiles - xcd_begin : per_xcd;
+    }
+    auto to_logical = [&](int64_t j) -> int64_t {
+        if (!windowed) return xcd_begin + j;
+        return ((j / group_span) * kNumXcd + xcd) * group_span + j % group_span;
+    };
 
-    struct TileInfo { int expert; int nt; int64_t row0; int rows_valid; };
+    const int KT = p.K / BK;
+    struct TileInfo { int expert; int nt; int64_t row0; int rows_valid; int64_t k_begin; int kt; };
     auto locate = [&](int64_t logical) -> TileInfo {
-        const int64_t group_span = (int64_t)kGroupM * p.n_tiles;
         const int64_t group = logical / group_span;
         const int first_m = (int)(group * kGroupM);
         const int gsize = total_m - first_m < kGroupM ? total_m - first_m : kGroupM;
@@ -797,6 +850,18 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             const int64_t left = (e_hi > e_lo ? e_hi : e_lo) - t.row0;
             t.rows_valid = (int)(left < BM ? left : BM);
         }
+        t.k_begin = 0;
+        t.kt = KT;
+        if (windowed) {
+            // whole pairs of K-slices, at least two pairs, inside the operands' columns
+            const int e = __builtin_amdgcn_readfirstlane(t.expert);
+            const int64_t lo = p.k_window[e], hi = p.k_window[e + 1];
+            int64_t kt = ((hi > lo ? hi - lo : 0) + 2 * BK - 1) / (2 * BK) * 2;
+            kt = kt < 4 ? 4 : kt;
+            kt = kt > KT / 2 * 2 ? KT / 2 * 2 : kt;
+            t.kt = (int)kt;
+            t.k_begin = clamp_i64(lo, 0, (int64_t)p.K - kt * BK);
+        }
         return t;
     };
 
@@ -833,7 +898,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     static_assert(!SWIGLU || (BN / 2) % (16 * NW) == 0, "a DMA instruction must not straddle gate and up rows");
     auto make_ptrs = [&](const TileInfo& t, const int64_t* ridx) {
         const int expert = __builtin_amdgcn_readfirstlane(t.expert);
-        xbase = p.a + (int64_t)expert * p.a_stride_e * ESIZE;
+        const int64_t k_begin = KWIN ? t.k_begin : 0;
+        xbase = p.a + ((int64_t)expert * p.a_stride_e + k_begin) * ESIZE;
         const int n0 = t.nt * BN_OUT;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
@@ -845,12 +911,24 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             const bool up = SWIGLU && i * NW * 16 >= BN / 2;
-            int n = n0 + wrow[i] - (up ? BN / 2 : 0);
-            n = n < p.N ? n : p.N - 1;
-            wbase[i] = (up ? p.b2 : p.b) + (int64_t)expert * p.b_se * ESIZE;
-            woff[i] = (uint32_t)((int64_t)n * p.b_sn * ESIZE) + wsw[i];
+            if constexpr (WTR) {
+                // instruction i of this wave: rows 4*wave + lane/16 of column block i, LDS position lane%16
+                const int kr = 4 * wave + (lane >> 4);
+                const int c = (lane & 15) ^ (4 * (lane >> 4));
+                int n = n0 + (SWIGLU ? 0 : i * (BN / 2)) + 8 * c;
+                n = n + 8 <= p.N ? n : p.N - 8;
+                wbase[i] = (up ? p.b2 : p.b) + ((int64_t)expert * p.b_se + k_begin * p.b_sk) * ESIZE;
+                woff[i] = (uint32_t)(((int64_t)kr * p.b_sk + n) * ESIZE);
+            } else {
+                int n = n0 + wrow[i] - (up ? BN / 2 : 0);
+                n = n < p.N ? n : p.N - 1;
+                wbase[i] = (up ? p.b2 : p.b) + ((int64_t)expert * p.b_se + k_begin) * ESIZE;
+                woff[i] = (uint32_t)((int64_t)n * p.b_sn * ESIZE) + wsw[i];
+            }
         }
     };
+    // bytes between the weight rows of consecutive K-slices
+    const int64_t wstep = WTR ? (int64_t)BK * p.b_sk * ESIZE : 64;
     // one K-slice into slot sa; in pair mode also the following slice into slot sb, the two
     // 64-byte halves of every row's 128 bytes requested by adjacent instructions
     auto issue = [&](int kt, int sa, int sb) {
@@ -862,10 +940,11 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             dma16(xbase + koff, xoff[i], abase + (i * NW + wave) * 1024);
             if (PAIR) dma16(xbase + koff + 64, xoff[i], bbase + (i * NW + wave) * 1024);
         }
+        const int64_t wkoff = (int64_t)kt * wstep;
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
-            dma16(wbase[i] + koff, woff[i], abase + BM * 64 + (i * NW + wave) * 1024);
-            if (PAIR) dma16(wbase[i] + koff + 64, woff[i], bbase + BM * 64 + (i * NW + wave) * 1024);
+            dma16(wbase[i] + wkoff, woff[i], abase + BM * 64 + (i * NW + wave) * 1024);
+            if (PAIR) dma16(wbase[i] + wkoff + wstep, woff[i], bbase + BM * 64 + (i * NW + wave) * 1024);
         }
     };
 
@@ -879,20 +958,30 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     }
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) xfrag_row[fm] = wm * TM + fm * 32 + (lane & 31);
+    // WTR: byte offset, inside the weight part of a slot, of this lane's first transposing read
+    // of fragment fn (rows 8*khalf + l16/4 of the slice's first 16; +1024: the next 4 rows)
+    int wtr_off[FN];
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+        const int l16 = lane & 15;
+        const int frag0 = wfrag_row[fn] - (lane & 31);                       // first tile column of the fragment
+        const int ncol = frag0 % (BN / 2) + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);
+        const int row = 8 * khalf + (l16 >> 2);
+        wtr_off[fn] = (frag0 / (BN / 2)) * 8192 + row * 256 + (((ncol >> 3) ^ (4 * (l16 >> 2))) << 4) + (ncol & 7) * 2;
+    }
 
-    const int KT = p.K / BK;
-    int64_t logical = xcd_begin + slot;
-    if (logical >= xcd_end) return;
-    const int my_tiles = (int)((xcd_end - logical + nslots - 1) / nslots);
-    const int total_items = my_tiles * KT;
+    if (slot >= xcd_count) return;
+    const int my_tiles = (int)((xcd_count - slot + nslots - 1) / nslots);
+    // 4-slot ring: every item of the block; paired ring: issue_next only starts the first tile
+    const int total_items = PAIR ? 4 : my_tiles * KT;
 
     // The block's work is one flat stream of K-slices ("items"): KT per tile, tile after
     // tile.  Item i lives in ring slot i % STAGES.  The issue side runs ahead of the compute
     // side and crosses tile boundaries on its own; it only needs the row pointers of the
     // tile it is in, the compute side only the TileInfo for the epilogue.
-    TileInfo cur = locate(logical);         // tile being computed
+    TileInfo cur = locate(to_logical(slot));   // tile being computed
     TileInfo nxt = cur;                     // tile after it (located one tile ahead)
-    int64_t ilogical = logical;
+    int64_t ilogical = slot;                // its number among the XCD's tiles
     int ikt = 0;                            // next K-slice to issue inside the issue tile
     int issued = 0;                         // items issued so far
     int islot = 0;                          // issued % STAGES
@@ -928,18 +1017,18 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     // waves backs up the CU's one address path and every wave sits in its issue, unable to
     // start MFMAs, until its own instructions are through.
     uint32_t part_a = 0, part_b = 0;
-    int64_t part_koff = 0;
+    int64_t part_koff = 0, part_wkoff = 0;
     auto issue_part = [&](int j) {          // j is a compile-time constant after unrolling
-        const uint8_t* base = (j < XI ? xbase : wbase[j >= XI ? j - XI : 0]) + part_koff;
+        const uint8_t* base = j < XI ? xbase + part_koff : wbase[j >= XI ? j - XI : 0] + part_wkoff;
         const uint32_t voff = j < XI ? xoff[j < XI ? j : 0] : woff[j >= XI ? j - XI : 0];
         const uint32_t off = (j < XI ? (j * NW + wave) * 1024 : BM * 64 + ((j - XI) * NW + wave) * 1024);
         dma16(base, voff, part_a + off);
-        dma16(base + 64, voff, part_b + off);
+        dma16(base + (j < XI ? (int64_t)64 : wstep), voff, part_b + off);
     };
     auto prefetch_next = [&]() {            // once per tile, early: locate the next tile and
         ilogical += nslots;                 // start fetching its source-row indices
-        if (ilogical < xcd_end) {
-            nxt = locate(ilogical);
+        if (ilogical < xcd_count) {
+            nxt = locate(to_logical(ilogical));
             fetch_rows(nxt, ridx_next);
         }
     };
@@ -967,6 +1056,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             for (int j = 0; j < FM; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        // SWIGLU: the counted wait that ends the epilogue does not settle every reload there (the
+        // second wave half reloads, before the epilogue, values only the first half keeps using);
+        // this one does, and after that long epilogue it finds little still in flight.
+        if (PAIR && FP8) wait_vmcnt<0>();
         if (tile_i > 0) prefetch_next();
 
         auto mma_slice = [&]() {
@@ -1031,8 +1124,20 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 const uint8_t* sw = sx + BM * 64;
                 const int chunk = 2 * sub + khalf;
 #pragma unroll
-                for (int fn = 0; fn < FN; ++fn)
-                    wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
+                for (int fn = 0; fn < FN; ++fn) {
+                    if constexpr (WTR) {
+                        typedef __attribute__((ext_vector_type(4))) short s16x4;
+                        typedef __attribute__((ext_vector_type(8))) short s16x8;
+                        typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+                        const uint8_t* a = sw + wtr_off[fn] + sub * 4096;     // 16 rows of 256 bytes on
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)a);
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(a + 1024));
+                        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                        wf[fn] = __builtin_bit_cast(bf16x8, both);
+                    } else {
+                        wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
+                    }
+                }
 #pragma unroll
                 for (int fm = 0; fm < FM; ++fm)
                     xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
@@ -1080,6 +1185,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 part_b = lds_base + islot * TL::STAGE_BYTES;
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
                 part_koff = (int64_t)ikt * 64;
+                part_wkoff = WTR ? (int64_t)ikt * wstep : part_koff;
                 ikt += 2;
                 load_block(wfb, xfb, s1, 1);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1097,7 +1203,14 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             // the issue side runs 4 items ahead: it enters the next tile 4 items before the end
             auto tile_steps = [&](auto half_c) {
-                for (int kt = 0; kt < KT - 4; kt += 2) double_step(half_c, std::false_type{});
+                const int tile_kt = KWIN ? cur.kt : KT;
+                // The first double step stands outside the loop, and every wave runs it in the
+                // second half's form (issue after A', vmcnt(0) before it): that explicit wait,
+                // which finds nothing young in flight, also settles whatever the compiler still
+                // counts as pending from the tile's set-up or the last epilogue (spill reloads,
+                // the row-index loads).  Left pending, their waits land inside the loop, where
+                // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
+                for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{});
                 make_ptrs(nxt, ridx_next);
                 ikt = 0;
                 double_step(half_c, std::false_type{});
@@ -1176,6 +1289,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 part_b = lds_base + islot * TL::STAGE_BYTES;
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
                 part_koff = (int64_t)ikt * 64;
+                part_wkoff = WTR ? (int64_t)ikt * wstep : part_koff;
                 ikt += 2;
                 load_x1(qx1, s1);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1191,7 +1305,14 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 cslot = s2;
             };
             auto tile_steps = [&](auto half_c) {
-                for (int kt = 0; kt < KT - 4; kt += 2) double_step(half_c, std::false_type{});
+                const int tile_kt = KWIN ? cur.kt : KT;
+                // The first double step stands outside the loop, and every wave runs it in the
+                // second half's form (issue after A', vmcnt(0) before it): that explicit wait,
+                // which finds nothing young in flight, also settles whatever the compiler still
+                // counts as pending from the tile's set-up or the last epilogue (spill reloads,
+                // the row-index loads).  Left pending, their waits land inside the loop, where
+                // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
+                for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{});
                 make_ptrs(nxt, ridx_next);
                 ikt = 0;
                 double_step(half_c, std::false_type{});
@@ -1277,11 +1398,11 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
 int compute_units();   // CUs of the current device (gemm_api.hip)
 int lds_per_block();   // largest LDS allocation of one block on the current device (gemm_api.hip)
 
-template <typename TL, bool FP8, int EPI>
+template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false>
 int launch_ring_cfg(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
-    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI>;
+    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN>;
     static bool attr_done = false;
     if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
     // persistent: one block per CU (the LDS footprint admits no second one), a multiple of
@@ -1299,6 +1420,25 @@ int launch_ring(const GemmParams& p, hipStream_t stream) {
     const int slices = p.K / (FP8 ? 64 : 32);
     const bool pair_ok = slices % 2 == 0 && slices >= 4 && p.total_rows < ((int64_t)1 << 31) &&
                          lds_per_block() >= TileRing5::LDS_BYTES;
+    // contraction windows: only the paired ring follows them, and only whole pairs of slices
+    const int pair_elems = FP8 ? 128 : 64;
+    const bool window_ok = !p.k_window || (p.k_window_multiple >= pair_elems && p.k_window_multiple % pair_elems == 0);
+    if (p.b_sn == 1 && p.b_sk != 1) {      // N-contiguous weights in place (the caller checked pair_ok's terms)
+        if constexpr (!FP8) {
+            if (p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI, true>(p, stream);
+            return launch_ring_cfg<TileRing5W, FP8, EPI, true>(p, stream);
+        }
+        return fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: no in-place path for these weights");
+    }
+    if (p.k_window) {                      // built for the weight gradient: bf16, no epilogue
+        if constexpr (!FP8 && EPI == FMOE_EPI_NONE) {
+            if (pair_ok && window_ok && p.E <= TileRing5::kMaxExperts)
+                return launch_ring_cfg<TileRing5, FP8, EPI, false, true>(p, stream);
+            if (pair_ok && window_ok && p.E <= TileRing5W::kMaxExperts)
+                return launch_ring_cfg<TileRing5W, FP8, EPI, false, true>(p, stream);
+        }
+        return launch_gemm<TileBig, FP8 ? kDtE4m3 : kDtBf16, EPI, true, false>(p, stream);
+    }
     if (pair_ok && p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI>(p, stream);
     if (pair_ok && p.E <= TileRing5W::kMaxExperts) return launch_ring_cfg<TileRing5W, FP8, EPI>(p, stream);
     return launch_ring_cfg<TileRing4, FP8, EPI>(p, stream);

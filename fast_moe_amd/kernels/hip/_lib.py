@@ -14,11 +14,13 @@ LIB_PATH = os.path.join(_PKG_DIR, "libfastmoe_hip.so")
 
 FMOE_F32, FMOE_BF16, FMOE_E4M3 = 0, 1, 2
 EPI_NONE, EPI_SILU, EPI_SWIGLU = 0, 1, 2
+PLAN_NONE, PLAN_RING, PLAN_STAGED, PLAN_STAGED_SHORT, PLAN_ELEMENT = -1, 0, 1, 2, 3
 
 # every symbol include/fast_moe_amd.h declares
 EXPORTED_SYMBOLS = (
     "fmoe_version", "fmoe_last_error", "fmoe_route_workspace_bytes", "fmoe_route_topk",
-    "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_combine",
+    "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_grouped_gemm_plan",
+    "fmoe_combine",
     "fmoe_silu_mul", "fmoe_transpose_last2", "fmoe_jagged_transpose", "fmoe_segment_colsum",
     "fmoe_swiglu_bwd", "fmoe_combine_bwd",
 )
@@ -77,6 +79,8 @@ def load() -> ctypes.CDLL:
                                          c_int, c_void_p]
     lib.fmoe_grouped_gemm.restype = c_int
     lib.fmoe_grouped_gemm.argtypes = [POINTER(GemmDesc), c_void_p]
+    lib.fmoe_grouped_gemm_plan.restype = c_int
+    lib.fmoe_grouped_gemm_plan.argtypes = [POINTER(GemmDesc), POINTER(c_int)]
     lib.fmoe_combine.restype = c_int
     lib.fmoe_combine.argtypes = [c_void_p, c_int, c_int64, c_int, c_int64, c_int64, c_void_p, c_void_p,
                                  c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_int, c_void_p]

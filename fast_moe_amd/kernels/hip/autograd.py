@@ -25,14 +25,19 @@ from . import ops
 from ._lib import EPI_NONE, EPI_SWIGLU
 
 
+_WINDOW_MULTIPLE = 64    # two 64-byte K-slices of bf16: what the LDS-ring GEMM steps by
+
+
 def _pad_layout(offsets: torch.Tensor, total_rows: int) -> Tuple[torch.Tensor, int]:
-    """Per-expert row counts rounded up to 8 -> (padded prefix [E+1], host-side bound of its end)."""
+    """Per-expert row counts rounded up to whole multiples of 64, at least 128 -> (padded prefix
+    [E+1], host-side bound of its end)."""
+    m = _WINDOW_MULTIPLE
     lengths = (offsets[1:] - offsets[:-1]).clamp_min(0)
-    padded = (lengths + 7) // 8 * 8
+    padded = ((lengths + m - 1) // m * m).clamp_min(2 * m)
     pad_offsets = torch.zeros_like(offsets)
     pad_offsets[1:] = torch.cumsum(padded, 0)
     E = offsets.numel() - 1
-    bound = (total_rows + 8 * E + 63) // 64 * 64
+    bound = (total_rows + 2 * m * E + m - 1) // m * m
     return pad_offsets, bound
 
 
@@ -69,7 +74,7 @@ class _WgradOperand:
         rows = torch.arange(E * N, device=dev, dtype=torch.int64) % N
         b = self.a_t.t().unsqueeze(0).expand(E, self.bound, Kin)                               # B[e, k, n'] = a_t[n', k]
         dw = ops.grouped_gemm(seg, dout_t, b, total_rows=E * N, row_index=rows, index_div=1, epilogue=EPI_NONE,
-                              k_window=self.pad_offsets)
+                              k_window=self.pad_offsets, k_window_multiple=_WINDOW_MULTIPLE)
         return dw.view(E, N, Kin)
 
 

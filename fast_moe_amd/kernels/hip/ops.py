@@ -212,16 +212,10 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     if offsets.numel() != E + 1:
         raise ValueError(f"grouped_gemm: offsets must have E+1={E + 1} entries")
     a = _rows_contiguous(a)
-    # N-contiguous weights of a useful size: one transposing copy buys the streaming kernel
-    # (the element-load kernel that reads them in place is correct but an order of magnitude slower)
     if k_window is not None:
         k_window = _i64("k_window", k_window)
         if k_window.numel() != E + 1:
             raise ValueError(f"grouped_gemm: k_window must have E+1={E + 1} entries")
-    elif b.stride(2) == 1 and b.stride(1) != 1 and K % 16 == 0 and N % 8 == 0 and total_rows * N >= (1 << 22):
-        b = to_k_contiguous(b)
-        if b2 is not None:
-            b2 = to_k_contiguous(b2)
     offsets = _i64("offsets", offsets)
     if row_index is not None:
         row_index = _i64("row_index", row_index).view(-1)
@@ -292,9 +286,27 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.k_window_multiple = k_window_multiple if k_window is not None else 0
     if aux is not None:
         d.aux, d.aux2, d.aux_stride_row = aux[0].data_ptr(), aux[1].data_ptr(), aux[0].stride(0)
-    rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
+    lib = _lib.load()
+    # N-contiguous weights of a useful size that only the element-load kernel would read in
+    # place (correct, but an order of magnitude slower): one transposing copy buys a streaming kernel
+    if (k_window is None and b.stride(2) == 1 and b.stride(1) != 1 and K % 16 == 0 and N % 8 == 0
+            and gemm_plan(d) == _lib.PLAN_ELEMENT and total_rows * N >= (1 << 22)):
+        b = to_k_contiguous(b)
+        d.b = b.data_ptr()
+        d.b_stride_e, d.b_stride_k, d.b_stride_n = b.stride()
+        if b2 is not None:
+            b2 = to_k_contiguous(b2)
+            d.b2 = b2.data_ptr()
+    rc = lib.fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
     _lib.check(rc, "fmoe_grouped_gemm")
     return out
+
+
+def gemm_plan(d: GemmDesc) -> int:
+    """The kernel fmoe_grouped_gemm would run for this descriptor (one of _lib.PLAN_*)."""
+    plan = ctypes.c_int(0)
+    _lib.check(_lib.load().fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)), "fmoe_grouped_gemm_plan")
+    return plan.value
 
 
 # ------------------------------------------------------------------ combine

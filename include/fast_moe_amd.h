@@ -205,6 +205,20 @@ typedef struct fmoe_gemm_desc {
 
 int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);
 
+/* Which kernel fmoe_grouped_gemm would run for this descriptor on the current device
+ * (no launch).  The Triton reference leaves this choice to its autotuner
+ * (kernels/triton/triton_moe.py:146-183); here it is a pure function of the descriptor, so
+ * a caller can see beforehand whether its weight layout is read in place by a streaming
+ * kernel or only by the element-load kernel, and tests can name the path they cover. */
+enum fmoe_gemm_plan {
+    FMOE_PLAN_NONE = -1,          /* nothing to do (no rows)                                */
+    FMOE_PLAN_RING = 0,           /* persistent LDS-ring kernel, 256 x 256 tiles            */
+    FMOE_PLAN_STAGED = 1,         /* register-staged kernel, 256 x 256 tiles                */
+    FMOE_PLAN_STAGED_SHORT = 2,   /* register-staged kernel, 64 x 256 tiles (few rows per expert) */
+    FMOE_PLAN_ELEMENT = 3         /* element loads: any strides, any alignment              */
+};
+int fmoe_grouped_gemm_plan(const fmoe_gemm_desc* desc, int* plan);
+
 /* ------------------------------------------------------------------ combine */
 
 /*

@@ -387,7 +387,7 @@ def test_full_size_c3_c4_sampled_rows(fp8):
         assert torch.equal(out[pos[(4, e)]], out[pos[(5, e)]])
 
 
-def test_n_contiguous_weights_take_the_transposing_fast_path():
+def test_n_contiguous_weights_and_the_transposing_copy():
     """[E, K, N]-contiguous weights (the layout of kernels/tests/moe_test.py:205-209) of a useful
     size are transposed once on the device and then streamed; the result equals the in-place
     element-load kernel's and the oracle's."""
@@ -500,3 +500,43 @@ def test_swiglu_pre_activation_outputs(L, E, K, Din, Dout, dtype, bias):
     assert torch.equal(aux[0], g) and torch.equal(aux[1], u)
     with pytest.raises(ValueError, match="SWIGLU"):
         ops.grouped_gemm(off, x, w, bias=b, aux=aux, **kw, **sc[0])
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,epi", [
+    (8192, 8, 2, 512, 384, "none"),
+    (8192, 8, 2, 512, 384, "swiglu"),
+    (4096, 16, 4, 256, 200, "none"),       # N tail: 200 columns of a 256-column tile
+    (4096, 16, 4, 256, 72, "swiglu"),      # N tail inside the gate / up halves
+    (20000, 200, 2, 128, 128, "swiglu"),   # register tables with 4 entries
+    (3000, 4, 2, 1408, 2048, "none"),      # the input-gradient shape of the layer
+])
+def test_ring_kernel_reads_n_contiguous_weights_in_place(L, E, K, Din, Dout, epi):
+    """[E, K, N]-contiguous weights (the reference tests' default layout, and what the input-gradient
+    GEMM multiplies by): the plan says RING, and the result is bit for bit the one from the same
+    weights stored K-contiguous."""
+    from fast_moe_amd.kernels.hip import _lib, ops
+    r = make_routing(L, E, K, seed=L + 1)
+    x = dev(randn((L, Din), 1))
+    w, wp = (dev(weights(E, Din, Dout, s, True, scale=Din ** -0.5)) for s in (2, 3))
+    b, bp = dev(randn((E, Dout), 4)), dev(randn((E, Dout), 5))
+    assert w.is_contiguous()
+    wk, wpk = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (w, wp))
+    kw = dict(total_rows=L * K, row_index=dev(r["index"]), index_div=K, bias=b)
+    if epi == "swiglu":
+        kw.update(bias2=bp, epilogue=_lib.EPI_SWIGLU)
+    off = dev(r["offsets"])
+    seen = []
+    real_plan = ops.gemm_plan
+    ops.gemm_plan = lambda d: seen.append(real_plan(d)) or seen[-1]
+    try:
+        out = ops.grouped_gemm(off, x, w, b2=wp if epi == "swiglu" else None, **kw)
+    finally:
+        ops.gemm_plan = real_plan
+    assert seen == [_lib.PLAN_RING]
+    ref = ops.grouped_gemm(off, x, wk, b2=wpk if epi == "swiglu" else None, **kw)
+    assert torch.equal(out, ref)
+    # a view with a larger row pitch (columns of a wider tensor) is read in place as well
+    wide = torch.zeros((E, Din, Dout + 24), dtype=BF16, device="cuda")
+    wide[:, :, 8:8 + Dout] = w
+    if epi == "none":
+        assert torch.equal(ops.grouped_gemm(off, x, wide[:, :, 8:8 + Dout], **kw), ref)
