@@ -125,7 +125,9 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
 // Rounding points follow the reference's bf16 path: GEMM result (+bias) rounded to bf16,
 // SiLU rounded to bf16, product rounded to bf16; e4m3 operands: (acc / (s_a * s_w)) rounded,
 // then the bias added in bf16.
-template <int FM, int FN, int TM, int TN, bool FP8, int EPI>
+// ALWAYS_VEC: the caller has checked p.vec_store (the ring kernel is only chosen with it), so
+// the element-store path is not even compiled in.
+template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
                                               int lane) {
@@ -141,8 +143,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     wn = __builtin_amdgcn_readfirstlane(wn);
     row0 = (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) |
                      (uint32_t)__builtin_amdgcn_readfirstlane((int)row0));
-    const uint32_t out_lane = (uint32_t)(lane & 31) * (uint32_t)p.out_stride * 2u + (uint32_t)khalf * 16u;
-    const uint32_t aux_lane = (uint32_t)(lane & 31) * (uint32_t)p.aux_stride * 2u + (uint32_t)khalf * 16u;
+    // (computed afresh at every store from a copy of the lane number the compiler cannot see
+    // through: hoisted out of the loops it becomes a 64-bit offset that is spilled and reloaded,
+    // with a full vmcnt(0) wait, before every single store)
+    auto lane_offset = [&](int64_t stride) -> uint32_t {
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return (uint32_t)(l & 31) * (uint32_t)stride * 2u + (uint32_t)(l >> 5) * 16u;
+    };
     float rsa[FM];
     bool row_ok[FM];
 #pragma unroll
@@ -150,7 +158,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         const int tile_row = wm * TM + fm * 32 + (lane & 31);
         row_ok[fm] = tile_row < rows_valid;
         rsa[fm] = 1.0f;
-        if (FP8) rsa[fm] = 1.0f / p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))];
+        if (FP8) rsa[fm] = __builtin_amdgcn_rcpf(p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))]);
     }
     // the bias-free form (FastMoE's SwiGLU experts, every fp8 call without bias) skips the adds
     auto run = [&](auto has_bias_c, auto has_aux_c) {
@@ -170,11 +178,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     for (int j = 0; j < 4; ++j) {
                         const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
                         const int nc = n < p.N ? n : p.N - 1;
-                        rsw[fn][gp][q][j] = FP8 ? 1.0f / p.b_scale[(int64_t)expert * p.N + nc] : 1.0f;
-                        rsw2[fn][gp][q][j] = (FP8 && SWIGLU) ? 1.0f / p.b2_scale[(int64_t)expert * p.N + nc] : 1.0f;
+                        // (v_rcp_f32 is exact on the powers of two the reference's scales are)
+                        rsw[fn][gp][q][j] = FP8 ? __builtin_amdgcn_rcpf(p.b_scale[(int64_t)expert * p.N + nc]) : 1.0f;
+                        rsw2[fn][gp][q][j] =
+                            (FP8 && SWIGLU) ? __builtin_amdgcn_rcpf(p.b2_scale[(int64_t)expert * p.N + nc]) : 1.0f;
                         bv[fn][gp][q][j] = HAS_BIAS && p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
                         bv2[fn][gp][q][j] = (HAS_BIAS && SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
                     }
+        __builtin_amdgcn_sched_barrier(0);
         // rows outermost: the stores that complete a row's 128-byte line follow each other
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
@@ -209,8 +220,9 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                             o[q][j] = y;
                         }
                     // base: first element of the 32-row block's first row (wave-uniform)
-                    auto store = [&](const float (&val)[2][4], uint16_t* base, uint32_t lane_off, int64_t stride) {
-                        if (p.vec_store) {
+                    auto store = [&](const float (&val)[2][4], uint16_t* base, int64_t stride) {
+                        if (ALWAYS_VEC || p.vec_store) {
+                            const uint32_t lane_off = lane_offset(stride);
                             // pair the quads of the two lane halves: low lanes end up with columns
                             // nq..nq+7, high lanes with nq+8..nq+15 of their row
                             const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(val[0][0], val[0][1]),
@@ -233,11 +245,14 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         }
                     };
                     const int64_t block_row = row0 + wm * TM + fm * 32;
-                    store(o, p.out + block_row * p.out_stride, out_lane, p.out_stride);
+                    store(o, p.out + block_row * p.out_stride, p.out_stride);
                     if (HAS_AUX) {
-                        store(pg, p.aux + block_row * p.aux_stride, aux_lane, p.aux_stride);
-                        store(pu, p.aux2 + block_row * p.aux_stride, aux_lane, p.aux_stride);
+                        store(pg, p.aux + block_row * p.aux_stride, p.aux_stride);
+                        store(pu, p.aux2 + block_row * p.aux_stride, p.aux_stride);
                     }
+                    // one column group at a time: interleaving the groups for more parallelism
+                    // is what runs the scheduler out of registers here
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
@@ -1348,7 +1363,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         const TileInfo done = cur;
         cur = nxt;      // valid when another tile follows (nxt was located at this tile's start)
 
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                 done.rows_valid, wm, wn, lane);
     }
     wait_vmcnt<0>();    // nothing may still be on its way into this block's LDS when it ends
