@@ -96,6 +96,12 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {   // v_cvt_pk_
 __device__ __forceinline__ float rbf(float a) {   // round to bf16 and back
     return (float)(__bf16)a;
 }
+// the same for two values with one conversion instruction
+__device__ __forceinline__ void rbf2(float& a, float& b) {
+    const uint32_t pk = pack_bf16(a, b);
+    a = __uint_as_float(pk << 16);
+    b = __uint_as_float(pk & 0xffff0000u);
+}
 
 // SiLU on 8 packed bf16 with the rounding of F.silu on a bf16 tensor
 __device__ __forceinline__ u32x4 silu_bf16x8(u32x4 v) {
@@ -195,29 +201,65 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                 for (int gp = 0; gp < 2; ++gp) {
                     const int nq = col0 + fn * 32 + 16 * gp;
                     float o[2][4], pg[2][4], pu[2][4];
+                    // two columns at a time: one conversion instruction rounds a pair
 #pragma unroll
                     for (int q = 0; q < 2; ++q)
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) {
+                        for (int j = 0; j < 4; j += 2) {
                             const int v = 4 * (2 * gp + q) + j;
-                            float y = acc[fn][fm][v];
-                            float y2 = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
+                            float ya = acc[fn][fm][v], yb = acc[fn][fm][v + 1];
+                            float ua = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
+                            float ub = SWIGLU ? acc[fn + FN / 2][fm][v + 1] : 0.0f;
                             if (FP8) {
-                                y = rbf(y * (rsa[fm] * rsw[fn][gp][q][j]));
-                                if (HAS_BIAS && p.bias) y = rbf(y + bv[fn][gp][q][j]);
+                                ya *= rsa[fm] * rsw[fn][gp][q][j];
+                                yb *= rsa[fm] * rsw[fn][gp][q][j + 1];
+                                rbf2(ya, yb);
+                                if (HAS_BIAS && p.bias) {
+                                    ya += bv[fn][gp][q][j];
+                                    yb += bv[fn][gp][q][j + 1];
+                                    rbf2(ya, yb);
+                                }
                                 if (SWIGLU) {
-                                    y2 = rbf(y2 * (rsa[fm] * rsw2[fn][gp][q][j]));
-                                    if (HAS_BIAS && p.bias2) y2 = rbf(y2 + bv2[fn][gp][q][j]);
+                                    ua *= rsa[fm] * rsw2[fn][gp][q][j];
+                                    ub *= rsa[fm] * rsw2[fn][gp][q][j + 1];
+                                    rbf2(ua, ub);
+                                    if (HAS_BIAS && p.bias2) {
+                                        ua += bv2[fn][gp][q][j];
+                                        ub += bv2[fn][gp][q][j + 1];
+                                        rbf2(ua, ub);
+                                    }
                                 }
                             } else {
-                                y = rbf(HAS_BIAS ? y + bv[fn][gp][q][j] : y);
-                                if (SWIGLU) y2 = rbf(HAS_BIAS ? y2 + bv2[fn][gp][q][j] : y2);
+                                if (HAS_BIAS) {
+                                    ya += bv[fn][gp][q][j];
+                                    yb += bv[fn][gp][q][j + 1];
+                                }
+                                rbf2(ya, yb);
+                                if (SWIGLU) {
+                                    if (HAS_BIAS) {
+                                        ua += bv2[fn][gp][q][j];
+                                        ub += bv2[fn][gp][q][j + 1];
+                                    }
+                                    rbf2(ua, ub);
+                                }
                             }
-                            pg[q][j] = y;
-                            pu[q][j] = y2;
-                            if (EPI == FMOE_EPI_SILU) y = fast_silu_f32(y);
-                            if (SWIGLU) y = rbf(fast_silu_f32(y)) * y2;
-                            o[q][j] = y;
+                            pg[q][j] = ya;
+                            pg[q][j + 1] = yb;
+                            pu[q][j] = ua;
+                            pu[q][j + 1] = ub;
+                            if (EPI == FMOE_EPI_SILU) {
+                                ya = fast_silu_f32(ya);
+                                yb = fast_silu_f32(yb);
+                            }
+                            if (SWIGLU) {
+                                ya = fast_silu_f32(ya);
+                                yb = fast_silu_f32(yb);
+                                rbf2(ya, yb);
+                                ya *= ua;
+                                yb *= ub;
+                            }
+                            o[q][j] = ya;
+                            o[q][j + 1] = yb;
                         }
                     // base: first element of the 32-row block's first row (wave-uniform)
                     auto store = [&](const float (&val)[2][4], uint16_t* base, int64_t stride) {
@@ -1074,7 +1116,6 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         // SWIGLU: the counted wait that ends the epilogue does not settle every reload there (the
         // second wave half reloads, before the epilogue, values only the first half keeps using);
         // this one does, and after that long epilogue it finds little still in flight.
-        if (PAIR && FP8) wait_vmcnt<0>();
         if (tile_i > 0) prefetch_next();
 
         auto mma_slice = [&]() {
