@@ -132,8 +132,9 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
 // SiLU rounded to bf16, product rounded to bf16; e4m3 operands: (acc / (s_a * s_w)) rounded,
 // then the bias added in bf16.
 // ALWAYS_VEC: the caller has checked p.vec_store (the ring kernel is only chosen with it), so
-// the element-store path is not even compiled in.
-template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false>
+// the element-store path is not even compiled in.  ROWS32: total_rows < 2^31 (the paired ring's
+// condition), so row numbers and row_index values fit 32 bits.
+template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false, bool ROWS32 = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
                                               int lane) {
@@ -161,10 +162,36 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     bool row_ok[FM];
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
-        const int tile_row = wm * TM + fm * 32 + (lane & 31);
-        row_ok[fm] = tile_row < rows_valid;
+        row_ok[fm] = wm * TM + fm * 32 + (lane & 31) < rows_valid;
         rsa[fm] = 1.0f;
-        if (FP8) rsa[fm] = __builtin_amdgcn_rcpf(p.a_scale[source_row(p, row0 + (row_ok[fm] ? tile_row : 0))]);
+    }
+    if (FP8) {
+        // the activation scales of this lane's rows: all index loads, then all scale loads (two
+        // memory latencies, not two per row block)
+        typedef typename std::conditional<ROWS32, int32_t, int64_t>::type row_t;
+        row_t src[FM];
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm)
+            src[fm] = (row_t)(row0 + (row_ok[fm] ? wm * TM + fm * 32 + (lane & 31) : 0));
+        if (p.row_index) {
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) {
+                if (ROWS32) src[fm] = reinterpret_cast<const int32_t*>(p.row_index)[2 * (int64_t)src[fm]];   // low half
+                else src[fm] = (row_t)p.row_index[src[fm]];
+            }
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm)
+                src[fm] = p.index_shift >= 0 ? (src[fm] >> p.index_shift) : src[fm] / (row_t)p.index_div;
+        }
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) {
+            const row_t last = (row_t)(p.a_rows - 1);
+            src[fm] = src[fm] < 0 ? 0 : (src[fm] > last ? last : src[fm]);
+        }
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) rsa[fm] = p.a_scale[src[fm]];
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm) rsa[fm] = __builtin_amdgcn_rcpf(rsa[fm]);
     }
     // the bias-free form (FastMoE's SwiGLU experts, every fp8 call without bias) skips the adds
     auto run = [&](auto has_bias_c, auto has_aux_c) {
@@ -174,6 +201,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         // with nq = first column of register-quad pair gp of fragment fn
         float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
         const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
+        // with a bias, at least one of the two pointers is set: both loads go through a valid
+        // pointer and a select drops the value of a missing one (a branch per load would make
+        // every load wait for the one before)
+        const uint16_t* bias_a = p.bias ? p.bias : p.bias2;
+        const uint16_t* bias_b = p.bias2 ? p.bias2 : p.bias;
 #pragma unroll
         for (int fn = 0; fn < FN_OUT; ++fn)
 #pragma unroll
@@ -188,8 +220,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         rsw[fn][gp][q][j] = FP8 ? __builtin_amdgcn_rcpf(p.b_scale[(int64_t)expert * p.N + nc]) : 1.0f;
                         rsw2[fn][gp][q][j] =
                             (FP8 && SWIGLU) ? __builtin_amdgcn_rcpf(p.b2_scale[(int64_t)expert * p.N + nc]) : 1.0f;
-                        bv[fn][gp][q][j] = HAS_BIAS && p.bias ? bf16_bits_to_f32(p.bias[bias_row + nc]) : 0.0f;
-                        bv2[fn][gp][q][j] = (HAS_BIAS && SWIGLU && p.bias2) ? bf16_bits_to_f32(p.bias2[bias_row + nc]) : 0.0f;
+                        bv[fn][gp][q][j] = bv2[fn][gp][q][j] = 0.0f;
+                        if (HAS_BIAS) {
+                            const float a = bf16_bits_to_f32(bias_a[bias_row + nc]);
+                            bv[fn][gp][q][j] = p.bias ? a : 0.0f;
+                        }
+                        if (HAS_BIAS && SWIGLU) {
+                            const float b = bf16_bits_to_f32(bias_b[bias_row + nc]);
+                            bv2[fn][gp][q][j] = p.bias2 ? b : 0.0f;
+                        }
                     }
         __builtin_amdgcn_sched_barrier(0);
         // rows outermost: the stores that complete a row's 128-byte line follow each other
@@ -926,25 +965,27 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     // DMA instruction i of this wave fills LDS rows (i*NW + wave)*16 .. +15 of the X (or W)
     // part of a ring slot: lane l -> row + l/4, 16-byte position l%4, which holds global
     // chunk (l%4) ^ ((row >> 2) & 3) of that row's 64-byte K-slice (the read-side swizzle).
-    int xrow[XI], wrow[WI];
-    int xsw[XI], wsw[WI];
-#pragma unroll
-    for (int i = 0; i < XI; ++i) {
-        xrow[i] = (i * NW + wave) * 16 + (lane >> 2);
-        xsw[i] = (((lane & 3) ^ ((xrow[i] >> 2) & 3)) << 4);
-    }
-#pragma unroll
-    for (int i = 0; i < WI; ++i) {
-        wrow[i] = (i * NW + wave) * 16 + (lane >> 2);
-        wsw[i] = (((lane & 3) ^ ((wrow[i] >> 2) & 3)) << 4);
-    }
+    // These are needed twice per tile and cost a few VALU instructions: they are recomputed from
+    // a copy of the lane number the compiler cannot see through rather than kept in registers
+    // across the main loop, where the accumulators and fragments leave none to spare.
+    auto dma_row = [&](int i) -> int {          // LDS row of DMA instruction i for this lane
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return (i * NW + wave) * 16 + (l >> 2);
+    };
+    auto dma_swizzle = [&](int i) -> int {      // byte position inside the row's 64-byte slice
+        int l = lane;
+        asm volatile("" : "+v"(l));
+        return (((l & 3) ^ ((((i * NW + wave) * 16 + (l >> 2)) >> 2) & 3)) << 4);
+    };
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem;
 
     // source rows (row_index entries) of a tile, fetched ahead of the pointer computation
     auto fetch_rows = [&](const TileInfo& t, int64_t* ridx) {
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
-            const int64_t r = t.row0 + (xrow[i] < t.rows_valid ? xrow[i] : 0);
+            const int xr = dma_row(i);
+            const int64_t r = t.row0 + (xr < t.rows_valid ? xr : 0);
             ridx[i] = p.row_index ? p.row_index[r] : r;
         }
     };
@@ -963,7 +1004,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             int64_t s = ridx[i];
             if (p.row_index) s = p.index_shift >= 0 ? (s >> p.index_shift) : s / p.index_div;
             s = clamp_i64(s, 0, p.a_rows - 1);
-            xoff[i] = (uint32_t)(s * (p.a_stride_row * ESIZE)) + xsw[i];
+            xoff[i] = (uint32_t)(s * (p.a_stride_row * ESIZE)) + dma_swizzle(i);
         }
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
@@ -977,10 +1018,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 wbase[i] = (up ? p.b2 : p.b) + ((int64_t)expert * p.b_se + k_begin * p.b_sk) * ESIZE;
                 woff[i] = (uint32_t)(((int64_t)kr * p.b_sk + n) * ESIZE);
             } else {
-                int n = n0 + wrow[i] - (up ? BN / 2 : 0);
+                int n = n0 + dma_row(i) - (up ? BN / 2 : 0);
                 n = n < p.N ? n : p.N - 1;
                 wbase[i] = (up ? p.b2 : p.b) + ((int64_t)expert * p.b_se + k_begin) * ESIZE;
-                woff[i] = (uint32_t)((int64_t)n * p.b_sn * ESIZE) + wsw[i];
+                woff[i] = (uint32_t)((int64_t)n * p.b_sn * ESIZE) + dma_swizzle(i);
             }
         }
     };
@@ -1404,7 +1445,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         const TileInfo done = cur;
         cur = nxt;      // valid when another tile follows (nxt was located at this tile's start)
 
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                 done.rows_valid, wm, wn, lane);
     }
     wait_vmcnt<0>();    // nothing may still be on its way into this block's LDS when it ends
