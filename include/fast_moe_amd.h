@@ -194,7 +194,9 @@ typedef struct fmoe_gemm_desc {
                                 only an upper bound); values multiples of 8          */
     int32_t k_window_multiple; /* 0, or a promise of the caller: every window length is a
                                 multiple of this many elements and at least twice it
-                                (64 or more lets the LDS-ring kernel take the call)   */
+                                (64 or more lets the LDS-ring kernel take the call; a
+                                broken promise gives wrong sums, never an access outside
+                                the k columns of A and B)                              */
     int32_t reserved0;      /* 0                                                  */
     void* aux;              /* NULL, or with FMOE_EPI_SWIGLU [total_rows, n] in out_dtype:  */
     void* aux2;             /* receive A x B + bias (aux) and A x B2 + bias2 (aux2), the

@@ -88,6 +88,23 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     d.a_dtype = 0                                    # fp32 operands need an fp32 output
     assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
     assert b"fp32 for fp32 operands" in lib.fmoe_last_error()
+    # pre-activation outputs come in pairs and belong to the SWIGLU epilogue; the plan query runs the same checks
+    d.a_dtype, d.out_dtype = 1, 1
+    d.offsets = d.a = d.b = d.out = 64
+    d.a_rows, d.index_div, d.a_stride_row, d.out_stride_row = 16, 1, 8, 8
+    d.aux = 64
+    assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
+    assert b"aux and aux2 come together" in lib.fmoe_last_error()
+    d.aux2 = 64
+    assert lib.fmoe_grouped_gemm(ctypes.byref(d), None) == 1
+    assert b"SWIGLU pre-activations" in lib.fmoe_last_error()
+    plan = ctypes.c_int(7)
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1 and plan.value == 7
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), None) == 1
+    assert b"plan is NULL" in lib.fmoe_last_error()
+    d.aux = d.aux2 = None
+    d.total_rows = 0
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 0 and plan.value == -1
     # routing: K > E, K > 64, workspace too small
     args = [None] * 7
     assert lib.fmoe_route_topk(None, 0, 4, 8, 80, 1, *args, None, 0, None) == 1
