@@ -994,18 +994,23 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     const uint8_t* xbase = p.a;
     const uint8_t* wbase[WI];
     static_assert(!SWIGLU || (BN / 2) % (16 * NW) == 0, "a DMA instruction must not straddle gate and up rows");
-    auto make_ptrs = [&](const TileInfo& t, const int64_t* ridx) {
-        const int expert = __builtin_amdgcn_readfirstlane(t.expert);
-        const int64_t k_begin = KWIN ? t.k_begin : 0;
-        xbase = p.a + ((int64_t)expert * p.a_stride_e + k_begin) * ESIZE;
-        const int n0 = t.nt * BN_OUT;
+    // fetched row_index entries -> this lane's byte offsets into A
+    auto rows_to_offsets = [&](const int64_t* ridx, uint32_t* out) {
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             int64_t s = ridx[i];
             if (p.row_index) s = p.index_shift >= 0 ? (s >> p.index_shift) : s / p.index_div;
             s = clamp_i64(s, 0, p.a_rows - 1);
-            xoff[i] = (uint32_t)(s * (p.a_stride_row * ESIZE)) + dma_swizzle(i);
+            out[i] = (uint32_t)(s * (p.a_stride_row * ESIZE)) + dma_swizzle(i);
         }
+    };
+    auto make_ptrs = [&](const TileInfo& t, const uint32_t* row_offsets) {
+        const int expert = __builtin_amdgcn_readfirstlane(t.expert);
+        const int64_t k_begin = KWIN ? t.k_begin : 0;
+        xbase = p.a + ((int64_t)expert * p.a_stride_e + k_begin) * ESIZE;
+        const int n0 = t.nt * BN_OUT;
+#pragma unroll
+        for (int i = 0; i < XI; ++i) xoff[i] = row_offsets[i];
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             const bool up = SWIGLU && i * NW * 16 >= BN / 2;
@@ -1083,18 +1088,36 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int ikt = 0;                            // next K-slice to issue inside the issue tile
     int issued = 0;                         // items issued so far
     int islot = 0;                          // issued % STAGES
+    // EARLY_ROWS: the row indices of a tile are fetched two tiles ahead, before the epilogue of
+    // the tile in between, and turned into offsets at the start of the tile before theirs: by
+    // then they have long arrived, and no load the compiler knows of is in flight while the
+    // main loop runs (its wait for one would also drain the LDS-DMA stream, which it cannot
+    // see).  Otherwise they are fetched at the start of the tile before theirs and converted
+    // when the issue side gets there: two registers fewer across the main loop, which is what
+    // the e4m3 kernels, at the limit of the register file, need more.
+    constexpr bool EARLY_ROWS = !FP8;
     int64_t ridx_next[XI];
+    uint32_t xoff_next[XI];
 #pragma unroll
-    for (int i = 0; i < XI; ++i) ridx_next[i] = 0;
+    for (int i = 0; i < XI; ++i) {
+        ridx_next[i] = 0;
+        xoff_next[i] = 0;
+    }
     {
         int64_t r0[XI];
+        uint32_t x0[XI];
         fetch_rows(cur, r0);
-        make_ptrs(cur, r0);
+        rows_to_offsets(r0, x0);
+        make_ptrs(cur, x0);
     }
+    auto enter_next = [&]() {               // the issue side moves on to the next tile
+        if (!EARLY_ROWS) rows_to_offsets(ridx_next, xoff_next);
+        make_ptrs(nxt, xoff_next);
+    };
     auto issue_next = [&]() {
         if (issued >= total_items) return;
         if (ikt == KT) {                    // the issue side enters the next tile
-            make_ptrs(nxt, ridx_next);
+            enter_next();
             ikt = 0;
         }
         const int sa = islot;
@@ -1154,10 +1177,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             for (int j = 0; j < FM; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-        // SWIGLU: the counted wait that ends the epilogue does not settle every reload there (the
-        // second wave half reloads, before the epilogue, values only the first half keeps using);
-        // this one does, and after that long epilogue it finds little still in flight.
-        if (tile_i > 0) prefetch_next();
+        if (EARLY_ROWS) rows_to_offsets(ridx_next, xoff_next);      // the tile after this one
+        else if (tile_i > 0) prefetch_next();
 
         auto mma_slice = [&]() {
             const uint8_t* sx = smem + cslot * TL::STAGE_BYTES;
@@ -1308,7 +1329,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 // the row-index loads).  Left pending, their waits land inside the loop, where
                 // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{});
-                make_ptrs(nxt, ridx_next);
+                enter_next();
                 ikt = 0;
                 double_step(half_c, std::false_type{});
                 double_step(half_c, std::true_type{});
@@ -1410,7 +1431,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 // the row-index loads).  Left pending, their waits land inside the loop, where
                 // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{});
-                make_ptrs(nxt, ridx_next);
+                enter_next();
                 ikt = 0;
                 double_step(half_c, std::false_type{});
                 double_step(half_c, std::true_type{});
@@ -1443,7 +1464,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             landed = issued - 2;
         }
         const TileInfo done = cur;
-        cur = nxt;      // valid when another tile follows (nxt was located at this tile's start)
+        cur = nxt;          // valid when another tile follows
+        if (EARLY_ROWS) prefetch_next();    // nxt: the tile after that one; its row indices arrive during the epilogue
 
         gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                 done.rows_valid, wm, wn, lane);
