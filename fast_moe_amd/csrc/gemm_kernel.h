@@ -834,8 +834,12 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int total_m;
     // register tables: lane l of entry i describes expert 64 * i + l
     int r_first[NR], r_lo[NR], r_len[NR];     // first row tile, first row, rows
+    // KWIN: the tables are in order of decreasing contraction window (the cost of an expert's
+    // tiles), r_exp tells which expert sits at a position: dealing groups of tiles to the XCDs
+    // back and forth then balances them whatever order the experts' loads come in.
+    int r_exp[NR];
     if constexpr (PAIR) {
-        int run = 0;
+        int e_lo[NR], e_len[NR];
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             const int e = i * kWave + lane;
@@ -845,6 +849,56 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 const int64_t hi = clamp_i64(p.offsets[e + 1], 0, R);
                 len = hi > lo ? hi - lo : 0;
             }
+            e_lo[i] = (int)lo;
+            e_len[i] = (int)len;
+            r_exp[i] = e;
+        }
+        if constexpr (KWIN) {
+            int e_w[NR], rank[NR], s_lo[NR], s_len[NR];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int e = i * kWave + lane;
+                int64_t w = -1;                 // positions past the last expert sort to the end
+                if (e < p.E) w = clamp_i64(p.k_window[e + 1] - p.k_window[e], 0, (int64_t)p.K);
+                e_w[i] = (int)w;
+                rank[i] = 0;
+                s_lo[i] = s_len[i] = 0;
+            }
+            auto pick = [&](const int (&arr)[NR], int o) -> int {     // entry of expert o, wave-uniform
+                int v = arr[0];
+#pragma unroll
+                for (int i = 1; i < NR; ++i)
+                    if ((o >> 6) == i) v = arr[i];
+                return uniform_lane(v, o & 63);
+            };
+            for (int o = 0; o < p.E; ++o) {     // rank = number of experts that sort before this one
+                const int wo = pick(e_w, o);
+#pragma unroll
+                for (int i = 0; i < NR; ++i) {
+                    const int e = i * kWave + lane;
+                    rank[i] += (wo > e_w[i] || (wo == e_w[i] && o < e)) ? 1 : 0;
+                }
+            }
+            for (int o = 0; o < p.E; ++o) {     // expert o moves to position rank[o]
+                const int ro = pick(rank, o), lo = pick(e_lo, o), len = pick(e_len, o);
+#pragma unroll
+                for (int i = 0; i < NR; ++i)
+                    if ((ro >> 6) == i && lane == (ro & 63)) {
+                        r_exp[i] = o;
+                        s_lo[i] = lo;
+                        s_len[i] = len;
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                e_lo[i] = s_lo[i];
+                e_len[i] = s_len[i];
+            }
+        }
+        int run = 0;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const int64_t lo = e_lo[i], len = e_len[i];
             const int tiles = (int)((len + BM - 1) / BM);
             const int inc = wave_inclusive_scan(tiles);
             r_first[i] = run + inc - tiles;
@@ -878,8 +932,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     }
     // The tiles of an XCD, numbered 0 .. xcd_count-1.  Without a contraction window: one
     // contiguous range of the tile order (neighbouring tiles share operands in the XCD's L2).
-    // With one the cost of a tile follows its expert's row count, so whole groups go round
-    // robin over the XCDs instead (a contiguous range would hand one XCD all the long experts).
+    // With one the cost of a tile follows its expert's row count, so whole groups are dealt to
+    // the XCDs instead, back and forth (0..7, 7..0, ...): a contiguous range would hand one XCD
+    // all the long experts, and a plain round robin still favours the low XCDs when the experts
+    // come sorted by load.
     const int64_t total_tiles = (int64_t)total_m * p.n_tiles;
     const int nslots = gridDim.x / kNumXcd;
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
@@ -888,11 +944,16 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int64_t xcd_begin, xcd_count;
     if (windowed) {
         const int64_t n_groups = (total_m + kGroupM - 1) / kGroupM;
-        const int64_t mine = n_groups > xcd ? (n_groups - xcd + kNumXcd - 1) / kNumXcd : 0;
+        // rounds of 8 groups; in odd rounds XCD x takes position 7 - x
+        const int64_t full_rounds = n_groups / kNumXcd, rest = n_groups % kNumXcd;
+        const int pos_in_last = (full_rounds & 1) ? kNumXcd - 1 - xcd : xcd;
+        const int64_t mine = full_rounds + (pos_in_last < rest ? 1 : 0);
         xcd_begin = 0;
         xcd_count = mine * group_span;
-        if (mine > 0 && (n_groups - 1) % kNumXcd == xcd)   // the last group may be short
-            xcd_count -= n_groups * group_span - total_tiles;
+        const int64_t last = n_groups - 1;                  // the last group may be short
+        const int last_pos = (int)(last % kNumXcd);
+        const int last_xcd = ((last / kNumXcd) & 1) ? kNumXcd - 1 - last_pos : last_pos;
+        if (n_groups > 0 && last_xcd == xcd) xcd_count -= n_groups * group_span - total_tiles;
     } else {
         const int64_t per_xcd = (total_tiles + kNumXcd - 1) / kNumXcd;
         xcd_begin = xcd * per_xcd;
@@ -900,7 +961,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     }
     auto to_logical = [&](int64_t j) -> int64_t {
         if (!windowed) return xcd_begin + j;
-        return ((j / group_span) * kNumXcd + xcd) * group_span + j % group_span;
+        const int64_t round = j / group_span;
+        const int pos = (round & 1) ? kNumXcd - 1 - xcd : xcd;
+        return (round * kNumXcd + pos) * group_span + j % group_span;
     };
 
     const int KT = p.K / BK;
@@ -924,13 +987,13 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             }
             cnt = __builtin_amdgcn_readfirstlane(cnt);
             const int ri = cnt >> 6, rl = cnt & 63;
-            int vf = r_first[0], vl = r_lo[0], vn = r_len[0];
+            int vf = r_first[0], vl = r_lo[0], vn = r_len[0], ve = r_exp[0];
 #pragma unroll
             for (int i = 1; i < NR; ++i)
-                if (ri == i) { vf = r_first[i]; vl = r_lo[i]; vn = r_len[i]; }
+                if (ri == i) { vf = r_first[i]; vl = r_lo[i]; vn = r_len[i]; ve = r_exp[i]; }
             const int first = uniform_lane(vf, rl), lo = uniform_lane(vl, rl), len = uniform_lane(vn, rl);
             const int skip = (mt - first) * BM;
-            t.expert = cnt;
+            t.expert = KWIN ? uniform_lane(ve, rl) : cnt;
             t.row0 = (int64_t)lo + skip;
             const int left = len - skip;
             t.rows_valid = left < BM ? left : BM;
