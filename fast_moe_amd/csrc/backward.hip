@@ -129,8 +129,11 @@ __global__ __launch_bounds__(256) void jagged_transpose_tr_kernel(
     const int grp = lane >> 4, j = lane & 15;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
-        const int pb = 2 * wave + (it & 1), half = it >> 1;
-        const int cbase = 64 * half + 16 * grp;
+        // the four 16-lane groups of a wave take four consecutive row blocks of the same 16
+        // columns: their 16-byte stores fill 64 contiguous bytes of each column's line
+        const int unit = 4 * wave + it;
+        const int pb = 4 * (unit >> 3) + grp;
+        const int cbase = 16 * (unit & 7);
         // this lane's read address: row 8*pb + j/4 (+4 for the second read), columns cbase + 4*(j%4)..+3
         uint8_t* a = tile + (8 * pb + (j >> 2)) * ROWB + (cbase + 4 * (j & 3)) * 2;
         typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
