@@ -134,7 +134,14 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
                          d->total_rows < ((int64_t)1 << 31) && lds_per_block() >= TileRing5::LDS_BYTES &&
                          d->a_rows * d->a_stride_row * esize + (int64_t)d->k * esize < span32 &&
                          ((int64_t)d->k * d->b_stride_k + d->n) * esize < span32;
-    sel = ring_tr ? kSelRing : !fast ? kSelGeneric : ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
+    // a contraction window is followed by the paired ring only (bf16, no epilogue, whole pairs of
+    // slices as promised by the caller, register tables); otherwise by the register-staged kernel
+    const bool ring_window = !fp8 && d->epilogue == FMOE_EPI_NONE && (d->k / slice) % 2 == 0 && d->k / slice >= 4 &&
+                             d->k_window_multiple >= 2 * slice && d->k_window_multiple % (2 * slice) == 0 &&
+                             d->num_experts <= TileRing5W::kMaxExperts && d->total_rows < ((int64_t)1 << 31) &&
+                             lds_per_block() >= TileRing5::LDS_BYTES;
+    const bool take_ring = ring && (!d->k_window || ring_window);
+    sel = ring_tr ? kSelRing : !fast ? kSelGeneric : take_ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
     return FMOE_OK;
 }
 

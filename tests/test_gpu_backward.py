@@ -238,3 +238,35 @@ def test_big_shape_forward_and_backward_64bit_offsets():
     ref_dx = torch.einsum("tkn,tkdn->td", table.float()[rr % 64], w0.float()[ee])
     close(x.grad[toks.cuda()], ref_dx, "big-shape d_jagged", rtol=3e-2, atol_frac=2e-2)
     assert w.grad.shape == w.shape and torch.isfinite(w.grad.float()).all()
+
+
+@pytest.mark.parametrize("order", ["descending", "shuffled"])
+def test_windowed_gemm_ring_and_staged_agree(order):
+    """The weight-gradient GEMM (per-expert contraction window) on the LDS-ring kernel, taken when the
+    caller promises windows of whole slice pairs, against the register-staged kernel without the promise
+    and against a per-expert matmul; expert loads in two orders (the ring kernel reorders them inside)."""
+    from fast_moe_amd.kernels.hip import autograd as ag, ops
+    E, N, Kin = 12, 256, 384
+    g = torch.Generator().manual_seed(7)
+    lens = torch.tensor([900, 700, 513, 400, 256, 130, 64, 63, 1, 0, 300, 77])
+    if order == "shuffled":
+        lens = lens[torch.randperm(E, generator=g)]
+    offsets = torch.zeros(E + 1, dtype=torch.int64)
+    offsets[1:] = torch.cumsum(lens, 0)
+    R = int(offsets[-1])
+    x = (torch.randn(R, Kin, generator=g) * 0.5).to(BF16)
+    d = (torch.randn(R, N, generator=g) * 0.5).to(BF16)
+    op = ag._WgradOperand(x.cuda(), offsets.cuda(), R)
+    dt = ops.jagged_transpose(d.cuda(), offsets.cuda(), op.pad_offsets, op.bound)
+    seg = torch.arange(E + 1, device="cuda", dtype=torch.int64) * N
+    rows = torch.arange(E * N, device="cuda", dtype=torch.int64) % N
+    b = op.a_t.t().unsqueeze(0).expand(E, op.bound, Kin)
+    kw = dict(total_rows=E * N, row_index=rows, index_div=1, k_window=op.pad_offsets)
+    ring = ops.grouped_gemm(seg, dt, b, k_window_multiple=64, **kw)
+    staged = ops.grouped_gemm(seg, dt, b, **kw)
+    ref = torch.stack([d[offsets[e]:offsets[e + 1]].float().t() @ x[offsets[e]:offsets[e + 1]].float() for e in range(E)])
+    for out, what in ((ring, "ring"), (staged, "staged")):
+        got = out.view(E, N, Kin).float().cpu()
+        err = (got - ref).abs().max().item()
+        assert err <= 2e-2 * ref.abs().max().item(), (what, err)
+    assert torch.equal(ring.view(E, N, Kin)[lens == 0], torch.zeros_like(ring.view(E, N, Kin)[lens == 0]))
