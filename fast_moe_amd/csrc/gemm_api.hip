@@ -46,8 +46,10 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     FMOE_REQUIRE(d->offsets && d->a && d->b && d->out, "fmoe_grouped_gemm: NULL tensor pointer");
     FMOE_REQUIRE(d->a_rows >= 1, "fmoe_grouped_gemm: a_rows < 1");
     FMOE_REQUIRE(d->index_div >= 1, "fmoe_grouped_gemm: index_div < 1");
-    FMOE_REQUIRE(d->a_stride_row >= d->k, "fmoe_grouped_gemm: A row stride %lld < k %d",
-                 (long long)d->a_stride_row, d->k);
+    const bool row_indexed = d->a_stride_k > 1;      // A (and B) given with k as the row index
+    if (!row_indexed)
+        FMOE_REQUIRE(d->a_stride_row >= d->k, "fmoe_grouped_gemm: A row stride %lld < k %d",
+                     (long long)d->a_stride_row, d->k);
     FMOE_REQUIRE(d->out_stride_row >= d->n, "fmoe_grouped_gemm: out row stride %lld < n %d",
                  (long long)d->out_stride_row, d->n);
     const bool fp8 = d->a_dtype == FMOE_E4M3;
@@ -80,6 +82,7 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     p.a = (const uint8_t*)d->a;
     p.a_stride_row = d->a_stride_row;
     p.a_stride_e = d->a_stride_e;
+    p.a_sk = row_indexed ? d->a_stride_k : 1;
     p.a_scale = d->a_scale;
     p.b = (const uint8_t*)d->b;
     p.b2 = (const uint8_t*)d->b2;
@@ -141,6 +144,23 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
                              d->num_experts <= TileRing5W::kMaxExperts && d->total_rows < ((int64_t)1 << 31) &&
                              lds_per_block() >= TileRing5::LDS_BYTES;
     const bool take_ring = ring && (!d->k_window || ring_window);
+    if (row_indexed) {
+        // the weight gradient from the row-major tensors themselves: paired ring only
+        const bool ok = !fp8 && !f32 && d->epilogue == FMOE_EPI_NONE && d->k_window && !d->a_silu &&
+                        d->a_stride_row == 1 && d->b_stride_n == 1 && d->a_stride_e == 0 &&
+                        (d->a_stride_k % chunk) == 0 && (d->b_stride_k % chunk) == 0 && (d->b_stride_e % chunk) == 0 &&
+                        aligned16(d->a) && aligned16(d->b) && (d->total_rows % 8) == 0 && p.vec_store &&
+                        d->k_slack_rows >= 4 * slice && d->k >= 4 * slice &&
+                        d->num_experts <= TileRing5W::kMaxExperts && d->total_rows < ((int64_t)1 << 31) &&
+                        lds_per_block() >= TileRing5::LDS_BYTES &&
+                        ((int64_t)2 * slice * d->a_stride_k + d->total_rows) * esize < span32 &&
+                        ((int64_t)2 * slice * d->b_stride_k + d->n) * esize < span32;
+        FMOE_REQUIRE(ok, "fmoe_grouped_gemm: row-indexed operands (a_stride_k > 1) need bf16, no epilogue, a "
+                         "k_window, unit strides along A's rows and B's columns, 16-byte alignment, row counts "
+                         "in multiples of 8, k_slack_rows >= 128, E <= 256 and a 160 KB LDS");
+        sel = kSelRing;
+        return FMOE_OK;
+    }
     sel = ring_tr ? kSelRing : !fast ? kSelGeneric : take_ring ? kSelRing : big ? kSelStagedBig : kSelStagedSmall;
     return FMOE_OK;
 }

@@ -51,6 +51,7 @@ struct GemmParams {
     int64_t total_rows, a_rows;
     const uint8_t* a;
     int64_t a_stride_row, a_stride_e;   // elements
+    int64_t a_sk;                       // element stride of A along k (1 unless A is given transposed)
     const float* a_scale;
     const uint8_t* b;
     const uint8_t* b2;
@@ -803,11 +804,23 @@ __device__ __forceinline__ int uniform_lane(int v, int src_lane) {
 //
 // KWIN: every expert contracts over its own window of K (p.k_window): the weight-gradient
 // GEMM.  Paired ring only; windows are whole pairs of K-slices, at least two pairs.
-template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false>
+//
+// XTR (with WTR and KWIN): both operands are given with the contraction index as their row
+// index, A[m][k] = a[k * a_sk + m] and B[k][n] = b[k * b_sk + n]: the weight gradient straight
+// from the row-major tensors it contracts (row gradients and input rows, both [rows, columns]
+// with the rows of an expert contiguous), no transposed copies.  The activation part of a slot
+// gets the layout described for WTR.  Windows are arbitrary row ranges: the slices of a tile
+// cover the window rounded up to whole pairs (at least two), and in the last two double steps
+// the weight-side fragments are masked beyond the window's end.  The rows read past the end
+// belong to the next expert or, after the last one, to the slack the caller promises
+// (k_slack_rows >= 128 readable rows behind both operands, finite values).
+template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false>
 __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmParams p) {
     static_assert(!WTR || (TL::PAIR && !FP8 && TL::BN == 256 && TL::NW == 8),
                   "in-place N-contiguous weights: bf16, paired ring, 256-column tiles of 8 waves");
-    static_assert(!KWIN || (TL::PAIR && !WTR), "contraction windows: paired ring, K-contiguous weights");
+    static_assert(!KWIN || TL::PAIR, "contraction windows: paired ring");
+    static_assert(XTR ? (WTR && KWIN && TL::BM == 256 && EPI == FMOE_EPI_NONE) : !(KWIN && WTR),
+                  "row-indexed operands come together, with a window, and without an epilogue");
     constexpr int BM = TL::BM, BN = TL::BN, NW = TL::NW, STAGES = TL::STAGES;
     constexpr int FM = TL::FM, FN = TL::FN, TM = TL::TM, TN = TL::TN;
     constexpr bool PAIR = TL::PAIR;
@@ -967,7 +980,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     };
 
     const int KT = p.K / BK;
-    struct TileInfo { int expert; int nt; int64_t row0; int rows_valid; int64_t k_begin; int kt; };
+    struct TileInfo { int expert; int nt; int64_t row0; int rows_valid; int64_t k_begin; int kt; int m0; int klen; };
     auto locate = [&](int64_t logical) -> TileInfo {
         const int64_t group = logical / group_span;
         const int first_m = (int)(group * kGroupM);
@@ -994,6 +1007,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             const int first = uniform_lane(vf, rl), lo = uniform_lane(vl, rl), len = uniform_lane(vn, rl);
             const int skip = (mt - first) * BM;
             t.expert = KWIN ? uniform_lane(ve, rl) : cnt;
+            t.m0 = skip;
             t.row0 = (int64_t)lo + skip;
             const int left = len - skip;
             t.rows_valid = left < BM ? left : BM;
@@ -1011,7 +1025,18 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         }
         t.k_begin = 0;
         t.kt = KT;
-        if (windowed) {
+        t.klen = 0;
+        if constexpr (!PAIR) t.m0 = 0;
+        if constexpr (XTR) {
+            // any row range; whole pairs of K-slices, at least two pairs
+            const int e = __builtin_amdgcn_readfirstlane(t.expert);
+            const int64_t lo = clamp_i64(p.k_window[e], 0, (int64_t)p.K);
+            const int64_t hi = clamp_i64(p.k_window[e + 1], lo, (int64_t)p.K);
+            int64_t kt = (hi - lo + 2 * BK - 1) / (2 * BK) * 2;
+            t.kt = (int)(kt < 4 ? 4 : kt);
+            t.k_begin = lo;
+            t.klen = (int)(hi - lo);
+        } else if (windowed) {
             // whole pairs of K-slices, at least two pairs, inside the operands' columns
             const int e = __builtin_amdgcn_readfirstlane(t.expert);
             const int64_t lo = p.k_window[e], hi = p.k_window[e + 1];
@@ -1045,6 +1070,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 
     // source rows (row_index entries) of a tile, fetched ahead of the pointer computation
     auto fetch_rows = [&](const TileInfo& t, int64_t* ridx) {
+        if constexpr (XTR) return;          // rows are not indexed: make_ptrs needs the tile only
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             const int xr = dma_row(i);
@@ -1059,6 +1085,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     static_assert(!SWIGLU || (BN / 2) % (16 * NW) == 0, "a DMA instruction must not straddle gate and up rows");
     // fetched row_index entries -> this lane's byte offsets into A
     auto rows_to_offsets = [&](const int64_t* ridx, uint32_t* out) {
+        if constexpr (XTR) return;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             int64_t s = ridx[i];
@@ -1070,17 +1097,36 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     auto make_ptrs = [&](const TileInfo& t, const uint32_t* row_offsets) {
         const int expert = __builtin_amdgcn_readfirstlane(t.expert);
         const int64_t k_begin = KWIN ? t.k_begin : 0;
-        xbase = p.a + ((int64_t)expert * p.a_stride_e + k_begin) * ESIZE;
         const int n0 = t.nt * BN_OUT;
+        if constexpr (XTR) {
+            // instruction i of this wave: k rows 4*wave + lane/16 of row block i (128 tile rows),
+            // LDS position lane%16 holding chunk (lane%16) ^ 4*(lane/16)
+            xbase = p.a + k_begin * p.a_sk * ESIZE;
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            const int kr = 4 * wave + (l >> 4);
+            const int c = (l & 15) ^ (4 * (l >> 4));
 #pragma unroll
-        for (int i = 0; i < XI; ++i) xoff[i] = row_offsets[i];
+            for (int i = 0; i < XI; ++i) {
+                int m = t.m0 + i * (BM / 2) + 8 * c;
+                const int last = t.m0 + t.rows_valid - 8;       // rows per expert: a multiple of 8
+                m = m <= last ? m : (last > 0 ? last : 0);
+                xoff[i] = (uint32_t)(((int64_t)kr * p.a_sk + m) * ESIZE);
+            }
+        } else {
+            xbase = p.a + ((int64_t)expert * p.a_stride_e + k_begin) * ESIZE;
+#pragma unroll
+            for (int i = 0; i < XI; ++i) xoff[i] = row_offsets[i];
+        }
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             const bool up = SWIGLU && i * NW * 16 >= BN / 2;
             if constexpr (WTR) {
                 // instruction i of this wave: rows 4*wave + lane/16 of column block i, LDS position lane%16
-                const int kr = 4 * wave + (lane >> 4);
-                const int c = (lane & 15) ^ (4 * (lane >> 4));
+                int l = lane;
+                asm volatile("" : "+v"(l));
+                const int kr = 4 * wave + (l >> 4);
+                const int c = (l & 15) ^ (4 * (l >> 4));
                 int n = n0 + (SWIGLU ? 0 : i * (BN / 2)) + 8 * c;
                 n = n + 8 <= p.N ? n : p.N - 8;
                 wbase[i] = (up ? p.b2 : p.b) + ((int64_t)expert * p.b_se + k_begin * p.b_sk) * ESIZE;
@@ -1095,16 +1141,17 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     };
     // bytes between the weight rows of consecutive K-slices
     const int64_t wstep = WTR ? (int64_t)BK * p.b_sk * ESIZE : 64;
+    const int64_t xstep = XTR ? (int64_t)BK * p.a_sk * ESIZE : 64;
     // one K-slice into slot sa; in pair mode also the following slice into slot sb, the two
     // 64-byte halves of every row's 128 bytes requested by adjacent instructions
     auto issue = [&](int kt, int sa, int sb) {
         const uint32_t abase = lds_base + sa * TL::STAGE_BYTES;
         const uint32_t bbase = lds_base + sb * TL::STAGE_BYTES;
-        const int64_t koff = (int64_t)kt * 64;
+        const int64_t koff = (int64_t)kt * xstep;
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             dma16(xbase + koff, xoff[i], abase + (i * NW + wave) * 1024);
-            if (PAIR) dma16(xbase + koff + 64, xoff[i], bbase + (i * NW + wave) * 1024);
+            if (PAIR) dma16(xbase + koff + xstep, xoff[i], bbase + (i * NW + wave) * 1024);
         }
         const int64_t wkoff = (int64_t)kt * wstep;
 #pragma unroll
@@ -1134,6 +1181,16 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         const int ncol = frag0 % (BN / 2) + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);
         const int row = 8 * khalf + (l16 >> 2);
         wtr_off[fn] = (frag0 / (BN / 2)) * 8192 + row * 256 + (((ncol >> 3) ^ (4 * (l16 >> 2))) << 4) + (ncol & 7) * 2;
+    }
+    // XTR: the same for the activation fragments (tile rows wm*TM + fm*32 ..)
+    int xtr_off[FM];
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+        const int l16 = lane & 15;
+        const int frag0 = wm * TM + fm * 32;
+        const int ncol = frag0 % (BM / 2) + 16 * ((lane >> 4) & 1) + 4 * (l16 & 3);
+        const int row = 8 * khalf + (l16 >> 2);
+        xtr_off[fm] = (frag0 / (BM / 2)) * 8192 + row * 256 + (((ncol >> 3) ^ (4 * (l16 >> 2))) << 4) + (ncol & 7) * 2;
     }
 
     if (slot >= xcd_count) return;
@@ -1207,7 +1264,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         const uint32_t voff = j < XI ? xoff[j < XI ? j : 0] : woff[j >= XI ? j - XI : 0];
         const uint32_t off = (j < XI ? (j * NW + wave) * 1024 : BM * 64 + ((j - XI) * NW + wave) * 1024);
         dma16(base, voff, part_a + off);
-        dma16(base + (j < XI ? (int64_t)64 : wstep), voff, part_b + off);
+        dma16(base + (j < XI ? xstep : wstep), voff, part_b + off);
     };
     auto prefetch_next = [&]() {            // once per tile, early: locate the next tile and
         ilogical += nslots;                 // start fetching its source-row indices
@@ -1300,28 +1357,45 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             // something to fetch (past the end of the block's stream it re-reads the last
             // tile's rows into slots nobody looks at), and everything that depends on the
             // wave's half is a template parameter.
-            auto load_block = [&](bf16x8 (&wf)[FN], bf16x8 (&xf)[FM], int slot_i, int sub) {
+            // two transposing reads: this lane's 8 k values of one column, 16 rows of 256 bytes
+            // (one MFMA's depth) starting at byte offset off of a slot part
+            auto read_tr = [&](const uint8_t* a) -> bf16x8 {
+                typedef __attribute__((ext_vector_type(4))) short s16x4;
+                typedef __attribute__((ext_vector_type(8))) short s16x8;
+                typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)a);
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(a + 1024));
+                const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                return __builtin_bit_cast(bf16x8, both);
+            };
+            // item: the slice's number inside the tile; mask_c: zero the weight-side values whose
+            // k lies at or beyond the end of the tile's window (XTR, the tile's last slices)
+            auto load_block = [&](bf16x8 (&wf)[FN], bf16x8 (&xf)[FM], int slot_i, int sub, int item, auto mask_c) {
+                constexpr bool MASK = XTR && decltype(mask_c)::value;
                 const uint8_t* sx = smem + slot_i * TL::STAGE_BYTES;
                 const uint8_t* sw = sx + BM * 64;
                 const int chunk = 2 * sub + khalf;
 #pragma unroll
                 for (int fn = 0; fn < FN; ++fn) {
-                    if constexpr (WTR) {
-                        typedef __attribute__((ext_vector_type(4))) short s16x4;
-                        typedef __attribute__((ext_vector_type(8))) short s16x8;
-                        typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
-                        const uint8_t* a = sw + wtr_off[fn] + sub * 4096;     // 16 rows of 256 bytes on
-                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)a);
-                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(a + 1024));
-                        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                        wf[fn] = __builtin_bit_cast(bf16x8, both);
-                    } else {
-                        wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
-                    }
+                    if constexpr (WTR) wf[fn] = read_tr(sw + wtr_off[fn] + sub * 4096);
+                    else wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
                 }
 #pragma unroll
-                for (int fm = 0; fm < FM; ++fm)
-                    xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
+                for (int fm = 0; fm < FM; ++fm) {
+                    if constexpr (XTR) xf[fm] = read_tr(sx + xtr_off[fm] + sub * 4096);
+                    else xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
+                }
+                if constexpr (MASK) {
+                    // register i of a fragment holds k = first + 2i, first + 2i + 1
+                    const int left = cur.klen - (item * BK + 16 * sub + 8 * khalf);
+                    u32x4 m;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        m[i] = left >= 2 * i + 2 ? 0xffffffffu : (left == 2 * i + 1 ? 0x0000ffffu : 0u);
+#pragma unroll
+                    for (int fn = 0; fn < FN; ++fn)
+                        wf[fn] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, wf[fn]) & m);
+                }
             };
             // the 8 MFMAs of a block, with the L parts of the pair being issued between them
             // when DMA is set.  The two waves of a SIMD (w and w + NW/2) issue in different
@@ -1347,16 +1421,17 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             // sched_barrier(0) pins the order "reads of the next block, then the MFMAs of this
             // one"; left alone the scheduler sinks the reads to just before their first use.
-            auto double_step = [&](auto half_c, auto last_c) {
+            int kitem = 0;                  // number, inside the tile, of the item in slot cslot
+            auto double_step = [&](auto half_c, auto last_c, auto mask_c) {
                 constexpr int HALF = decltype(half_c)::value;
                 constexpr bool LAST = decltype(last_c)::value;   // last of the tile: no fragments kept over the epilogue
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
                 const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
-                load_block(wfb, xfb, cslot, 1);
+                load_block(wfb, xfb, cslot, 1, kitem, mask_c);
                 __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfa, xfa, std::false_type{});
                 __builtin_amdgcn_sched_barrier(0);
-                load_block(wfa, xfa, s1, 0);
+                load_block(wfa, xfa, s1, 0, kitem + 1, mask_c);
                 __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfb, xfb, std::false_type{});
                 __builtin_amdgcn_sched_barrier(0);
@@ -1365,10 +1440,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
                 part_b = lds_base + islot * TL::STAGE_BYTES;
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
-                part_koff = (int64_t)ikt * 64;
+                part_koff = (int64_t)ikt * xstep;
                 part_wkoff = WTR ? (int64_t)ikt * wstep : part_koff;
                 ikt += 2;
-                load_block(wfb, xfb, s1, 1);
+                load_block(wfb, xfb, s1, 1, kitem + 1, mask_c);
                 __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfa, xfa, std::integral_constant<bool, HALF == 0>{});
                 __builtin_amdgcn_sched_barrier(0);
@@ -1376,32 +1451,28 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 if (HALF == 0) wait_vmcnt<2 * L>();
                 else wait_vmcnt<0>();
                 barrier();                  // A'
-                if (!LAST) load_block(wfa, xfa, s2, 0);
+                if (!LAST) load_block(wfa, xfa, s2, 0, kitem + 2, mask_c);
                 __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfb, xfb, std::integral_constant<bool, HALF == 1>{});
                 __builtin_amdgcn_sched_barrier(0);
                 cslot = s2;
+                kitem += 2;
             };
-            // the issue side runs 4 items ahead: it enters the next tile 4 items before the end
+            // the issue side runs 4 items ahead: it enters the next tile 4 items before the end;
+            // the last two double steps hold the end of an XTR tile's window and mask it
             auto tile_steps = [&](auto half_c) {
                 const int tile_kt = KWIN ? cur.kt : KT;
-                // The first double step stands outside the loop, and every wave runs it in the
-                // second half's form (issue after A', vmcnt(0) before it): that explicit wait,
-                // which finds nothing young in flight, also settles whatever the compiler still
-                // counts as pending from the tile's set-up or the last epilogue (spill reloads,
-                // the row-index loads).  Left pending, their waits land inside the loop, where
-                // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
-                for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{});
+                for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{}, std::false_type{});
                 enter_next();
                 ikt = 0;
-                double_step(half_c, std::false_type{});
-                double_step(half_c, std::true_type{});
+                double_step(half_c, std::false_type{}, std::true_type{});
+                double_step(half_c, std::true_type{}, std::true_type{});
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
                 wait_vmcnt<2 * L>();
                 barrier();
             }
-            load_block(wfa, xfa, cslot, 0);
+            load_block(wfa, xfa, cslot, 0, 0, std::true_type{});
             if (wave < NW / 2) tile_steps(std::integral_constant<int, 0>{});
             else tile_steps(std::integral_constant<int, 1>{});
         } else if constexpr (PAIR) {
@@ -1469,7 +1540,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
                 part_b = lds_base + islot * TL::STAGE_BYTES;
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
-                part_koff = (int64_t)ikt * 64;
+                part_koff = (int64_t)ikt * xstep;
                 part_wkoff = WTR ? (int64_t)ikt * wstep : part_koff;
                 ikt += 2;
                 load_x1(qx1, s1);
@@ -1580,11 +1651,11 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
 int compute_units();   // CUs of the current device (gemm_api.hip)
 int lds_per_block();   // largest LDS allocation of one block on the current device (gemm_api.hip)
 
-template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false>
+template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false>
 int launch_ring_cfg(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
-    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN>;
+    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN, XTR>;
     static bool attr_done = false;
     if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
     // persistent: one block per CU (the LDS footprint admits no second one), a multiple of
@@ -1605,6 +1676,13 @@ int launch_ring(const GemmParams& p, hipStream_t stream) {
     // contraction windows: only the paired ring follows them, and only whole pairs of slices
     const int pair_elems = FP8 ? 128 : 64;
     const bool window_ok = !p.k_window || (p.k_window_multiple >= pair_elems && p.k_window_multiple % pair_elems == 0);
+    if (p.a_sk != 1) {                     // both operands row-indexed (the caller checked the rest)
+        if constexpr (!FP8 && EPI == FMOE_EPI_NONE) {
+            if (p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI, true, true, true>(p, stream);
+            return launch_ring_cfg<TileRing5W, FP8, EPI, true, true, true>(p, stream);
+        }
+        return fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: row-indexed operands need bf16 and no epilogue");
+    }
     if (p.b_sn == 1 && p.b_sk != 1) {      // N-contiguous weights in place (the caller checked pair_ok's terms)
         if constexpr (!FP8) {
             if (p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI, true>(p, stream);

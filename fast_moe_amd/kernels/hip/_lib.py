@@ -42,10 +42,11 @@ class GemmDesc(ctypes.Structure):
         ("out", c_void_p), ("out_stride_row", c_int64),
         ("k_window", c_void_p),
         ("k_window_multiple", c_int32),
-        ("reserved0", c_int32),
+        ("k_slack_rows", c_int32),
         ("aux", c_void_p),
         ("aux2", c_void_p),
         ("aux_stride_row", c_int64),
+        ("a_stride_k", c_int64),
     ]
 
 

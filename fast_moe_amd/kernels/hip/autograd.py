@@ -52,19 +52,39 @@ def _reverse_from_index(index: torch.Tensor) -> torch.Tensor:
 
 
 class _WgradOperand:
-    """The input rows of the routed rows, transposed and zero padded per expert ([K_in, bound]),
-    with the padded layout it was written in: shared by the weight gradients of every weight
-    that multiplied the same input (SwiGLU's gate and up projections)."""
+    """The input rows of the routed rows as the weight-gradient GEMM wants them, shared by the
+    weight gradients of every weight that multiplied the same input (SwiGLU's gate and up
+    projections).  Preferred form: the rows themselves in expert order with slack behind them
+    (one gather copy when they are indexed), contracted in place with the row gradients.
+    Otherwise: transposed and zero padded per expert ([K_in, bound])."""
 
     def __init__(self, a_src: torch.Tensor, offsets: torch.Tensor, total_rows: int, *,
                  row_index: Optional[torch.Tensor] = None, index_div: int = 1, apply_silu: bool = False):
         self.offsets = offsets
-        self.pad_offsets, self.bound = _pad_layout(offsets, total_rows)
-        self.a_t = ops.jagged_transpose(a_src, offsets, self.pad_offsets, self.bound, row_index, index_div,
-                                        apply_silu)
+        self.args = (a_src, total_rows, row_index, index_div, apply_silu)
+        self.rows = None            # [total_rows, K_in] in expert order, with slack
+        self.a_t = None
+        if a_src.dtype == torch.bfloat16 and not apply_silu:
+            if row_index is None:
+                self.rows = a_src
+            else:
+                self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
+                torch.index_select(a_src, 0, torch.div(row_index, index_div, rounding_mode="floor"), out=self.rows)
+
+    def _transposed(self):
+        if self.a_t is None:
+            a_src, total_rows, row_index, index_div, apply_silu = self.args
+            self.pad_offsets, self.bound = _pad_layout(self.offsets, total_rows)
+            self.a_t = ops.jagged_transpose(a_src, self.offsets, self.pad_offsets, self.bound, row_index, index_div,
+                                            apply_silu)
 
     def weight_grad(self, dout: torch.Tensor) -> torch.Tensor:
         """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a(r)[k] -> [E, N, K_in]."""
+        if self.rows is not None:
+            dw = ops.jagged_weight_grad(dout, self.rows, self.offsets)
+            if dw is not None:
+                return dw
+        self._transposed()
         N = dout.shape[1]
         Kin = self.a_t.shape[0]
         E = self.offsets.numel() - 1

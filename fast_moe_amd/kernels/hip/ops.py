@@ -178,6 +178,60 @@ def to_k_contiguous(w: torch.Tensor) -> torch.Tensor:
     return dst.permute(0, 2, 1)
 
 
+# ------------------------------------------------------- rows with slack
+SLACK_ROWS = 128    # what fmoe_grouped_gemm asks for behind row-indexed operands
+
+
+def empty_rows(rows: int, cols: int, dtype: torch.dtype, device) -> torch.Tensor:
+    """[rows, cols] view of a buffer with SLACK_ROWS more rows behind it, those zeroed: what the
+    weight-gradient GEMM may read (and masks out) past an expert's last row."""
+    buf = torch.empty((rows + SLACK_ROWS, cols), dtype=dtype, device=device)
+    buf[rows:].zero_()
+    return buf[:rows]
+
+
+def slack_rows(t: torch.Tensor) -> int:
+    """Rows of t's row pitch that its storage holds behind its last row."""
+    if t.ndim != 2 or t.stride(1) != 1 or t.stride(0) < t.shape[1]:
+        return 0
+    have = t.untyped_storage().nbytes() // t.element_size() - t.storage_offset()
+    return max(0, (have - t.shape[1]) // t.stride(0) + 1 - t.shape[0]) if t.stride(0) > 0 else 0
+
+
+def jagged_weight_grad(dout: torch.Tensor, a_rows: torch.Tensor, offsets: torch.Tensor) -> Optional[torch.Tensor]:
+    """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a_rows[r, k] -> [E, N, K_in],
+    both operands read in place (fmoe_grouped_gemm with a_stride_k).  Returns None when the
+    operands do not qualify (dtype, alignment, no slack behind them): the caller then takes the
+    route over transposed copies."""
+    if dout.dtype != torch.bfloat16 or a_rows.dtype != torch.bfloat16 or dout.shape[0] != a_rows.shape[0]:
+        return None
+    R, N = dout.shape
+    Kin = a_rows.shape[1]
+    E = offsets.numel() - 1
+    ok = (dout.stride(1) == 1 and a_rows.stride(1) == 1 and N % 8 == 0 and Kin % 8 == 0 and E <= 256
+          and dout.stride(0) % 8 == 0 and a_rows.stride(0) % 8 == 0 and dout.data_ptr() % 16 == 0
+          and a_rows.data_ptr() % 16 == 0 and R >= 128 and E * N < (1 << 31)
+          and slack_rows(dout) >= SLACK_ROWS and slack_rows(a_rows) >= SLACK_ROWS)
+    if not ok:
+        return None
+    dev = dout.device
+    offsets = _i64("offsets", offsets)
+    seg = torch.arange(E + 1, device=dev, dtype=torch.int64) * N
+    out = torch.empty((E * N, Kin), dtype=torch.bfloat16, device=dev)
+    d = GemmDesc()
+    d.num_experts, d.n, d.k, d.index_div = E, Kin, R, 1
+    d.total_rows, d.a_rows = E * N, N
+    d.offsets = seg.data_ptr()
+    d.a, d.a_dtype, d.a_stride_row, d.a_stride_k = dout.data_ptr(), _DTYPE_CODE[dout.dtype], 1, dout.stride(0)
+    d.b, d.b_stride_e, d.b_stride_k, d.b_stride_n = a_rows.data_ptr(), 0, a_rows.stride(0), 1
+    d.epilogue, d.out_dtype = EPI_NONE, _DTYPE_CODE[torch.bfloat16]
+    d.out, d.out_stride_row = out.data_ptr(), Kin
+    d.k_window, d.k_slack_rows = offsets.data_ptr(), SLACK_ROWS
+    rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(dout))
+    _lib.check(rc, "fmoe_grouped_gemm")
+    return out.view(E, N, Kin)
+
+
 # -------------------------------------------------------------- grouped GEMM
 def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, total_rows: int,
                  row_index: Optional[torch.Tensor] = None, index_div: int = 1,
@@ -221,8 +275,8 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
         row_index = _i64("row_index", row_index).view(-1)
         if row_index.numel() != total_rows:
             raise ValueError("grouped_gemm: row_index must have total_rows entries")
-    if out is None:
-        out = torch.empty((total_rows, N), dtype=out_dtype, device=dev)
+    if out is None:    # (with slack: the output may become an operand of a weight-gradient GEMM)
+        out = empty_rows(total_rows, N, out_dtype, dev)
     elif (tuple(out.shape) != (total_rows, N) or out.dtype != out_dtype or out.device != dev
           or out.stride(1) != 1):
         raise ValueError(f"grouped_gemm: out must be {out_dtype} [{total_rows}, {N}] with contiguous rows")
@@ -408,8 +462,9 @@ def swiglu_bwd(g: torch.Tensor, u: Optional[torch.Tensor], dh: torch.Tensor):
         raise ValueError("swiglu_bwd: bf16 (or fp32) tensors of one shape expected")
     g, dh = g.contiguous(), dh.contiguous()
     u = None if u is None else u.contiguous()
-    dg = torch.empty_like(g)
-    du = None if u is None else torch.empty_like(g)
+    dg = empty_rows(g.shape[0], g.shape[1], g.dtype, g.device) if g.ndim == 2 else torch.empty_like(g)
+    du = None if u is None else (empty_rows(g.shape[0], g.shape[1], g.dtype, g.device) if g.ndim == 2
+                                 else torch.empty_like(g))
     rc = _lib.load().fmoe_swiglu_bwd(g.data_ptr(), _ptr(u), dh.data_ptr(), dg.data_ptr(), _ptr(du),
                                      _DTYPE_CODE[g.dtype], g.numel(), _stream(g))
     _lib.check(rc, "fmoe_swiglu_bwd")
@@ -448,7 +503,7 @@ def combine_bwd(dy: torch.Tensor, value: Optional[torch.Tensor], token_index: to
         value = _rows_contiguous(value)
         v_stride = value.stride(0)
         d_gates = torch.zeros((R,), dtype=torch.float32, device=dev)
-    d_value = torch.empty((R, D), dtype=dy.dtype, device=dev)
+    d_value = empty_rows(R, D, dy.dtype, dev)
     rc = _lib.load().fmoe_combine_bwd(
         dy.data_ptr(), _ptr(value) if need_gate_grad else None, _DTYPE_CODE[dy.dtype], T, K, D, v_stride,
         token_index.data_ptr(), _ptr(gates), g_code, g_cols, g_sr, g_sc, _ptr(gates_index), d_value.data_ptr(),

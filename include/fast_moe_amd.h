@@ -197,12 +197,22 @@ typedef struct fmoe_gemm_desc {
                                 (64 or more lets the LDS-ring kernel take the call; a
                                 broken promise gives wrong sums, never an access outside
                                 the k columns of A and B)                              */
-    int32_t reserved0;      /* 0                                                  */
+    int32_t k_slack_rows;   /* with a_stride_k: rows readable behind the last k row of A and of
+                                B (finite values; 128 or more)                       */
     void* aux;              /* NULL, or with FMOE_EPI_SWIGLU [total_rows, n] in out_dtype:  */
     void* aux2;             /* receive A x B + bias (aux) and A x B2 + bias2 (aux2), the
                                 two pre-activations the backward pass needs (the ALPHA and
                                 BETA outputs of kernels/triton/triton_moe.py:2316-2345) */
     int64_t aux_stride_row;
+    int64_t a_stride_k;     /* 0 / 1: A rows are contiguous along k.  > 1: both operands are given
+                                with the contraction index as their row index, A[m][k] =
+                                a[k*a_stride_k + m] (a_stride_row = 1) and B[k][n] = b[k*b_stride_k
+                                + n] (b_stride_n = 1, b_stride_e = 0), and k_window holds arbitrary
+                                row ranges: the weight gradient straight from the row gradients
+                                [rows, n_out] and the expert-sorted input rows [rows, n_in], with
+                                no transposed copies (bf16, FMOE_EPI_NONE, LDS-ring kernel only;
+                                row_index is not used; every expert's output row count a multiple
+                                of 8)                                                   */
 } fmoe_gemm_desc;
 
 int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);

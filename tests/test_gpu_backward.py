@@ -257,6 +257,7 @@ def test_windowed_gemm_ring_and_staged_agree(order):
     x = (torch.randn(R, Kin, generator=g) * 0.5).to(BF16)
     d = (torch.randn(R, N, generator=g) * 0.5).to(BF16)
     op = ag._WgradOperand(x.cuda(), offsets.cuda(), R)
+    op._transposed()                        # the route over transposed, zero padded copies
     dt = ops.jagged_transpose(d.cuda(), offsets.cuda(), op.pad_offsets, op.bound)
     seg = torch.arange(E + 1, device="cuda", dtype=torch.int64) * N
     rows = torch.arange(E * N, device="cuda", dtype=torch.int64) % N
@@ -270,3 +271,40 @@ def test_windowed_gemm_ring_and_staged_agree(order):
         err = (got - ref).abs().max().item()
         assert err <= 2e-2 * ref.abs().max().item(), (what, err)
     assert torch.equal(ring.view(E, N, Kin)[lens == 0], torch.zeros_like(ring.view(E, N, Kin)[lens == 0]))
+
+
+@pytest.mark.parametrize("lens", [
+    [900, 700, 513, 400, 256, 130, 64, 63, 1, 0, 300, 77],      # ragged, empty, tiny, not multiples of anything
+    [0, 0, 5, 0, 2000, 129, 0, 127],                            # leading empties, a window just over two slices
+    [128] * 70,                                                 # more than 64 experts: the 4-entry register tables
+])
+def test_weight_gradient_from_rows_in_place(lens):
+    """fmoe_grouped_gemm with a_stride_k: dW[e] = dout_e^T x_e read straight from the row-major tensors
+    (arbitrary row ranges, masked window ends, slack behind the last row), against per-expert matmuls."""
+    from fast_moe_amd.kernels.hip import ops
+    E, N, Kin = len(lens), 264, 392                             # N, Kin tails inside the 256-wide tiles
+    g = torch.Generator().manual_seed(11)
+    lens = torch.tensor(lens)
+    offsets = torch.zeros(E + 1, dtype=torch.int64)
+    offsets[1:] = torch.cumsum(lens, 0)
+    R = int(offsets[-1])
+    x = (torch.randn(R, Kin, generator=g) * 0.5).to(BF16)
+    d = (torch.randn(R, N, generator=g) * 0.5).to(BF16)
+    xg, dg = ops.empty_rows(R, Kin, BF16, "cuda"), ops.empty_rows(R, N, BF16, "cuda")
+    xg.copy_(x)
+    dg.copy_(d)
+    assert ops.slack_rows(xg) >= ops.SLACK_ROWS and ops.slack_rows(x.cuda()) == 0
+    out = ops.jagged_weight_grad(dg, xg, offsets.cuda())
+    assert out is not None and tuple(out.shape) == (E, N, Kin)
+    assert ops.jagged_weight_grad(d.cuda(), xg, offsets.cuda()) is None      # no slack behind dout: refused
+    ref = torch.stack([d[offsets[e]:offsets[e + 1]].float().t() @ x[offsets[e]:offsets[e + 1]].float() for e in range(E)])
+    got = out.float().cpu()
+    err = (got - ref).abs().max().item()
+    assert err <= 2e-2 * max(1.0, ref.abs().max().item()), err
+    assert torch.equal(got[lens == 0], torch.zeros_like(got[lens == 0]))
+    # garbage behind the rows of the last expert must not leak in: poison the slack with large finite values
+    xg2 = ops.empty_rows(R, Kin, BF16, "cuda")
+    xg2.copy_(x)
+    torch.as_strided(xg2, (ops.SLACK_ROWS, Kin), (Kin, 1), R * Kin).fill_(3.0e4)
+    out2 = ops.jagged_weight_grad(dg, xg2, offsets.cuda())
+    assert torch.equal(out2, out)
