@@ -64,10 +64,13 @@ class _WgradOperand:
         self.args = (a_src, total_rows, row_index, index_div, apply_silu)
         self.rows = None            # [total_rows, K_in] in expert order, with slack
         self.a_t = None
-        if a_src.dtype == torch.bfloat16 and not apply_silu:
-            if row_index is None:
+        if a_src.dtype == torch.bfloat16 and a_src.ndim == 2:
+            if row_index is None and not apply_silu:
                 self.rows = a_src
-            else:
+            elif row_index is None:             # SiLU with the rounding of F.silu on a bf16 tensor
+                self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
+                torch.ops.aten.silu.out(a_src, out=self.rows)
+            elif not apply_silu:
                 self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
                 torch.index_select(a_src, 0, torch.div(row_index, index_div, rounding_mode="floor"), out=self.rows)
 
