@@ -811,9 +811,9 @@ __device__ __forceinline__ int uniform_lane(int v, int src_lane) {
 // with the rows of an expert contiguous), no transposed copies.  The activation part of a slot
 // gets the layout described for WTR.  Windows are arbitrary row ranges: the slices of a tile
 // cover the window rounded up to whole pairs (at least two), and in the last two double steps
-// the weight-side fragments are masked beyond the window's end.  The rows read past the end
-// belong to the next expert or, after the last one, to the slack the caller promises
-// (k_slack_rows >= 128 readable rows behind both operands, finite values).
+// the fragments are masked beyond the window's end.  The rows read past the end belong to the
+// next expert or, after the last one, to the slack the caller promises (k_slack_rows >= 128
+// readable rows behind both operands; their contents do not matter).
 template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false>
 __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmParams p) {
     static_assert(!WTR || (TL::PAIR && !FP8 && TL::BN == 256 && TL::NW == 8),
@@ -1395,6 +1395,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 #pragma unroll
                     for (int fn = 0; fn < FN; ++fn)
                         wf[fn] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, wf[fn]) & m);
+                    // both sides: what lies behind the window need not even be finite
+#pragma unroll
+                    for (int fm = 0; fm < FM; ++fm)
+                        xf[fm] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, xf[fm]) & m);
                 }
             };
             // the 8 MFMAs of a block, with the L parts of the pair being issued between them

@@ -183,11 +183,9 @@ SLACK_ROWS = 128    # what fmoe_grouped_gemm asks for behind row-indexed operand
 
 
 def empty_rows(rows: int, cols: int, dtype: torch.dtype, device) -> torch.Tensor:
-    """[rows, cols] view of a buffer with SLACK_ROWS more rows behind it, those zeroed: what the
-    weight-gradient GEMM may read (and masks out) past an expert's last row."""
-    buf = torch.empty((rows + SLACK_ROWS, cols), dtype=dtype, device=device)
-    buf[rows:].zero_()
-    return buf[:rows]
+    """[rows, cols] view of a buffer with SLACK_ROWS more rows behind it: what the weight-gradient
+    GEMM may read (and masks out, whatever they hold) past an expert's last row."""
+    return torch.empty((rows + SLACK_ROWS, cols), dtype=dtype, device=device)[:rows]
 
 
 def slack_rows(t: torch.Tensor) -> int:

@@ -198,7 +198,7 @@ typedef struct fmoe_gemm_desc {
                                 broken promise gives wrong sums, never an access outside
                                 the k columns of A and B)                              */
     int32_t k_slack_rows;   /* with a_stride_k: rows readable behind the last k row of A and of
-                                B (finite values; 128 or more)                       */
+                                B (128 or more; what they hold does not matter)      */
     void* aux;              /* NULL, or with FMOE_EPI_SWIGLU [total_rows, n] in out_dtype:  */
     void* aux2;             /* receive A x B + bias (aux) and A x B2 + bias2 (aux2), the
                                 two pre-activations the backward pass needs (the ALPHA and

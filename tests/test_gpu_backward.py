@@ -302,9 +302,11 @@ def test_weight_gradient_from_rows_in_place(lens):
     err = (got - ref).abs().max().item()
     assert err <= 2e-2 * max(1.0, ref.abs().max().item()), err
     assert torch.equal(got[lens == 0], torch.zeros_like(got[lens == 0]))
-    # garbage behind the rows of the last expert must not leak in: poison the slack with large finite values
-    xg2 = ops.empty_rows(R, Kin, BF16, "cuda")
+    # what lies behind the rows of the last expert must not leak in: poison both slacks with NaN
+    xg2, dg2 = ops.empty_rows(R, Kin, BF16, "cuda"), ops.empty_rows(R, N, BF16, "cuda")
     xg2.copy_(x)
-    torch.as_strided(xg2, (ops.SLACK_ROWS, Kin), (Kin, 1), R * Kin).fill_(3.0e4)
-    out2 = ops.jagged_weight_grad(dg, xg2, offsets.cuda())
+    dg2.copy_(d)
+    torch.as_strided(xg2, (ops.SLACK_ROWS, Kin), (Kin, 1), R * Kin).fill_(float("nan"))
+    torch.as_strided(dg2, (ops.SLACK_ROWS, N), (N, 1), R * N).fill_(float("nan"))
+    out2 = ops.jagged_weight_grad(dg2, xg2, offsets.cuda())
     assert torch.equal(out2, out)
