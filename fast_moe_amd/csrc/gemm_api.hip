@@ -62,6 +62,11 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
         FMOE_REQUIRE(d->aux_stride_row >= d->n, "fmoe_grouped_gemm: aux row stride %lld < n %d",
                      (long long)d->aux_stride_row, d->n);
     }
+    const bool two = d->a2 != nullptr;               // out = a * b + a2 * b2
+    if (two)
+        FMOE_REQUIRE(d->b2 && d->k2 >= 1 && d->epilogue == FMOE_EPI_NONE && !d->k_window && !row_indexed,
+                     "fmoe_grouped_gemm: a2 needs b2 and k2, and goes with no epilogue and no k_window");
+    const int ktot = d->k + (two ? d->k2 : 0);
     if (fp8) {
         FMOE_REQUIRE(d->a_scale && d->b_scale, "fmoe_grouped_gemm: e4m3 operands need a_scale and b_scale");
         if (swiglu) FMOE_REQUIRE(d->b2_scale != nullptr, "fmoe_grouped_gemm: SWIGLU e4m3 needs b2_scale");
@@ -72,7 +77,9 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     p.row_index = d->row_index;
     p.E = d->num_experts;
     p.N = d->n;
-    p.K = d->k;
+    p.K = ktot;
+    p.a2 = (const uint8_t*)d->a2;
+    p.k_split = d->k;
     p.index_div = d->index_div;
     p.index_shift = -1;
     for (int s = 0; s < 31; ++s)
@@ -132,11 +139,18 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     const bool ring_tr = !fp8 && !f32 && big && !d->a_silu && !d->k_window && d->b_stride_n == 1 &&
                          d->b_stride_k != 1 && (d->b_stride_k % chunk) == 0 && (d->b_stride_e % chunk) == 0 &&
                          (d->a_stride_row % chunk) == 0 && (d->a_stride_e % chunk) == 0 && aligned16(d->a) &&
-                         aligned16(d->b) && (!swiglu || aligned16(d->b2)) && (d->k % (2 * slice)) == 0 &&
-                         d->k / slice >= 4 && p.vec_store && d->num_experts <= TileRing5W::kMaxExperts &&
+                         aligned16(d->b) && (!(swiglu || two) || aligned16(d->b2)) && (d->k % (2 * slice)) == 0 &&
+                         (ktot % (2 * slice)) == 0 && (!two || aligned16(d->a2)) &&
+                         ktot / slice >= 4 && p.vec_store && d->num_experts <= TileRing5W::kMaxExperts &&
                          d->total_rows < ((int64_t)1 << 31) && lds_per_block() >= TileRing5::LDS_BYTES &&
-                         d->a_rows * d->a_stride_row * esize + (int64_t)d->k * esize < span32 &&
-                         ((int64_t)d->k * d->b_stride_k + d->n) * esize < span32;
+                         d->a_rows * d->a_stride_row * esize + (int64_t)ktot * esize < span32 &&
+                         ((int64_t)ktot * d->b_stride_k + d->n) * esize < span32;
+    // the second product exists in that kernel only; a caller that is turned away runs two
+    // GEMMs and adds
+    if (two)
+        FMOE_REQUIRE(ring_tr, "fmoe_grouped_gemm: a2 * b2 is summed in only by the kernel that reads bf16 weights "
+                              "B[e][k][n] with n contiguous: k and k2 in multiples of 128, 16-byte alignment, "
+                              "96 or more rows per expert on average, E <= 256, a 160 KB LDS");
     // a contraction window is followed by the paired ring only (bf16, no epilogue, whole pairs of
     // slices as promised by the caller, register tables); otherwise by the register-staged kernel
     const bool ring_window = !fp8 && d->epilogue == FMOE_EPI_NONE && (d->k / slice) % 2 == 0 && d->k / slice >= 4 &&

@@ -70,6 +70,8 @@ struct GemmParams {
     uint16_t* aux;                      // SWIGLU: the two pre-activations, or null
     uint16_t* aux2;
     int64_t aux_stride;
+    const uint8_t* a2;                  // second product a2 * b2 summed into the same output, or null
+    int k_split;                        // ... whose contraction covers k in [k_split, K)
 };
 
 constexpr int kDtBf16 = 0, kDtE4m3 = 1, kDtF32 = 2;
@@ -1142,18 +1144,29 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     // bytes between the weight rows of consecutive K-slices
     const int64_t wstep = WTR ? (int64_t)BK * p.b_sk * ESIZE : 64;
     const int64_t xstep = XTR ? (int64_t)BK * p.a_sk * ESIZE : 64;
+    // A second product a2 * b2 continued in the same accumulators: the K-slices from split_kt on
+    // come from a2 and b2, addressed with the strides of a and b.  (A pair of slices never
+    // straddles the split: k_split is a whole number of pairs.)
+    constexpr bool SPLIT = WTR && PAIR && !FP8 && !SWIGLU && !KWIN && !XTR;
+    const int split_kt = SPLIT && p.a2 ? p.k_split / BK : 0x7fffffff;
+    const int64_t split_x = SPLIT && p.a2 ? (p.a2 - p.a) - (int64_t)split_kt * xstep : 0;
+    const int64_t split_w = SPLIT && p.a2 ? (p.b2 - p.b) - (int64_t)split_kt * wstep : 0;
     // one K-slice into slot sa; in pair mode also the following slice into slot sb, the two
     // 64-byte halves of every row's 128 bytes requested by adjacent instructions
     auto issue = [&](int kt, int sa, int sb) {
         const uint32_t abase = lds_base + sa * TL::STAGE_BYTES;
         const uint32_t bbase = lds_base + sb * TL::STAGE_BYTES;
-        const int64_t koff = (int64_t)kt * xstep;
+        int64_t koff = (int64_t)kt * xstep;
+        int64_t wkoff = (int64_t)kt * wstep;
+        if constexpr (SPLIT) {
+            koff += kt >= split_kt ? split_x : 0;
+            wkoff += kt >= split_kt ? split_w : 0;
+        }
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             dma16(xbase + koff, xoff[i], abase + (i * NW + wave) * 1024);
             if (PAIR) dma16(xbase + koff + xstep, xoff[i], bbase + (i * NW + wave) * 1024);
         }
-        const int64_t wkoff = (int64_t)kt * wstep;
 #pragma unroll
         for (int i = 0; i < WI; ++i) {
             dma16(wbase[i] + wkoff, woff[i], abase + BM * 64 + (i * NW + wave) * 1024);
@@ -1446,6 +1459,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 islot = islot + 1 == STAGES ? 0 : islot + 1;
                 part_koff = (int64_t)ikt * xstep;
                 part_wkoff = WTR ? (int64_t)ikt * wstep : part_koff;
+                if constexpr (SPLIT) {
+                    part_koff += ikt >= split_kt ? split_x : 0;
+                    part_wkoff += ikt >= split_kt ? split_w : 0;
+                }
                 ikt += 2;
                 load_block(wfb, xfb, s1, 1, kitem + 1, mask_c);
                 __builtin_amdgcn_sched_barrier(0);

@@ -47,6 +47,7 @@ class GemmDesc(ctypes.Structure):
         ("aux2", c_void_p),
         ("aux_stride_row", c_int64),
         ("a_stride_k", c_int64),
+        ("a2", c_void_p), ("k2", c_int32), ("reserved1", c_int32),
     ]
 
 

@@ -106,6 +106,11 @@ def _input_grad(drow_list, weights, offsets, reverse_index) -> torch.Tensor:
     R = drow_list[0].shape[0]
     n = len(drow_list)
     Kin = weights[0].shape[1]
+    if n == 2:      # both branches of a SwiGLU layer in one GEMM where the kernel allows
+        w0, w1 = (w.permute(0, 2, 1) for w in weights)
+        value = ops.grouped_gemm_sum2(offsets, drow_list[0], w0, drow_list[1], w1, total_rows=R)
+        if value is not None:
+            return ops.combine(value, reverse_index)
     value = torch.empty((n * R, Kin), dtype=drow_list[0].dtype, device=drow_list[0].device)
     for i, (d, w) in enumerate(zip(drow_list, weights)):
         ops.grouped_gemm(offsets, d, w.permute(0, 2, 1), total_rows=R, out=value[i * R:(i + 1) * R])

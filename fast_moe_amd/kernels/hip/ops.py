@@ -354,6 +354,41 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     return out
 
 
+def grouped_gemm_sum2(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, a2: torch.Tensor,
+                      b2: torch.Tensor, *, total_rows: int,
+                      out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``a @ b[e] + a2 @ b2[e]`` per expert in one pass, accumulated in fp32 and rounded once
+    (fmoe_gemm_desc.a2): a, a2 [rows, K], [rows, K2] bf16; b, b2 [E, K, N], [E, K2, N] with N
+    contiguous.  None when the operands do not qualify: the caller runs two GEMMs and adds."""
+    dev = _need_cuda("grouped_gemm_sum2", offsets, a, b, a2, b2)
+    E, K, N = b.shape
+    K2 = b2.shape[1]
+    if (any(t.dtype != torch.bfloat16 for t in (a, b, a2, b2)) or a.ndim != 2 or a2.ndim != 2
+            or a.shape != (total_rows, K) or a2.shape != (total_rows, K2) or b2.shape != (E, K2, N)
+            or a.stride(1) != 1 or a2.stride() != a.stride() or b2.stride() != b.stride() or total_rows == 0):
+        return None
+    offsets = _i64("offsets", offsets)
+    if out is None:
+        out = empty_rows(total_rows, N, torch.bfloat16, dev)
+    d = GemmDesc()
+    d.num_experts, d.n, d.k, d.index_div = E, N, K, 1
+    d.total_rows = d.a_rows = total_rows
+    d.offsets = offsets.data_ptr()
+    d.a, d.a2, d.k2 = a.data_ptr(), a2.data_ptr(), K2
+    d.a_dtype = d.out_dtype = _DTYPE_CODE[torch.bfloat16]
+    d.a_stride_row = a.stride(0)
+    d.b, d.b2 = b.data_ptr(), b2.data_ptr()
+    d.b_stride_e, d.b_stride_k, d.b_stride_n = b.stride()
+    d.epilogue = EPI_NONE
+    d.out, d.out_stride_row = out.data_ptr(), out.stride(0)
+    lib = _lib.load()
+    plan = ctypes.c_int(0)
+    if lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) != 0:
+        return None
+    _lib.check(lib.fmoe_grouped_gemm(ctypes.byref(d), _stream(a)), "fmoe_grouped_gemm")
+    return out
+
+
 def gemm_plan(d: GemmDesc) -> int:
     """The kernel fmoe_grouped_gemm would run for this descriptor (one of _lib.PLAN_*)."""
     plan = ctypes.c_int(0)

@@ -213,6 +213,18 @@ typedef struct fmoe_gemm_desc {
                                 no transposed copies (bf16, FMOE_EPI_NONE, LDS-ring kernel only;
                                 row_index is not used; every expert's output row count a multiple
                                 of 8)                                                   */
+    const void* a2;         /* NULL, or a second product summed into the same output:
+                                out = a * b + a2 * b2, with a2 [rows, k2] and b2 [E, k2, n] under
+                                the strides of a and b (so k2 = k unless the tensors are views of
+                                larger ones).  The input gradient of a SwiGLU layer,
+                                d_gate * W_gate + d_up * W_up, in one pass with one output; the
+                                reference runs two GEMMs, rounds each and adds
+                                (kernels/triton/triton_moe.py:2472-2500), here the sum is rounded
+                                once.  bf16, FMOE_EPI_NONE (bias allowed), weights with n
+                                contiguous (b_stride_n = 1), k and k2 in multiples of 128; other
+                                descriptors with a2 are turned away with FMOE_ERR_ARGUMENT */
+    int32_t k2;             /* contraction length of a2 * b2                                */
+    int32_t reserved1;
 } fmoe_gemm_desc;
 
 int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);

@@ -103,6 +103,10 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), None) == 1
     assert b"plan is NULL" in lib.fmoe_last_error()
     d.aux = d.aux2 = None
+    d.a2, d.k2 = 64, 128                     # a second product needs b2 and goes with no epilogue
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
+    assert b"a2 needs b2" in lib.fmoe_last_error()
+    d.a2, d.k2 = None, 0
     d.total_rows = 0
     assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 0 and plan.value == -1
     # routing: K > E, K > 64, workspace too small

@@ -310,3 +310,32 @@ def test_weight_gradient_from_rows_in_place(lens):
     torch.as_strided(dg2, (ops.SLACK_ROWS, N), (N, 1), R * N).fill_(float("nan"))
     out2 = ops.jagged_weight_grad(dg2, xg2, offsets.cuda())
     assert torch.equal(out2, out)
+
+
+@pytest.mark.parametrize("lens,K1,K2,N", [
+    ([300, 0, 1000, 128, 77, 515], 256, 256, 256),
+    ([4096, 640], 384, 384, 520),
+])
+def test_two_products_in_one_gemm(lens, K1, K2, N):
+    """out = a @ b + a2 @ b2 (the SwiGLU input gradient) in one pass: bit-identical to the same
+    kernel run on the operands concatenated along k, and close to fp32."""
+    from fast_moe_amd.kernels.hip import ops
+    E, R = len(lens), sum(lens)
+    offsets = torch.tensor([0] + lens).cumsum(0)
+    a, a2 = randn((R, K1), 1).to(BF16).cuda(), randn((R, K2), 2).to(BF16).cuda()
+    w, w2 = (randn((E, K, N), s, scale=0.05).to(BF16).cuda() for K, s in ((K1, 3), (K2, 4)))
+    out = ops.grouped_gemm_sum2(offsets.cuda(), a, w, a2, w2, total_rows=R)
+    assert out is not None, "shape chosen to qualify"
+    cat = ops.grouped_gemm(offsets.cuda(), torch.cat([a, a2], 1), torch.cat([w, w2], 1), total_rows=R)
+    assert torch.equal(out, cat)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if lo == hi:
+            continue
+        ref = a[lo:hi].float() @ w[e].float() + a2[lo:hi].float() @ w2[e].float()
+        close(out[lo:hi], ref, f"expert {e}", rtol=1e-2, atol_frac=4e-3)
+    # operands that do not qualify are declined, not mangled
+    assert ops.grouped_gemm_sum2(offsets.cuda(), a.float(), w.float(), a2.float(), w2.float(), total_rows=R) is None
+    wk = w.transpose(1, 2).contiguous().transpose(1, 2)      # k contiguous
+    wk2 = w2.transpose(1, 2).contiguous().transpose(1, 2)
+    assert ops.grouped_gemm_sum2(offsets.cuda(), a, wk, a2, wk2, total_rows=R) is None
