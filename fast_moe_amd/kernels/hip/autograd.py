@@ -168,6 +168,81 @@ class IndexSelectJaggedBmm(torch.autograd.Function):
         return None, None, d_jagged, d_w, d_b, d_wp, d_bp
 
 
+class IndexSelectJaggedGatingBmm(torch.autograd.Function):
+    """index_select_jagged_gating_bmm with two different inputs: silu(A Wa + ba) * (B Wb + bb)
+    (backward of kernels/triton/triton_moe.py:2839-2990)."""
+
+    @staticmethod
+    def forward(ctx, offsets, index, jagged_a, jagged_b, weight_a, weight_b, bias_a, bias_b):
+        R, K = index.numel(), index.shape[-1]
+        pre_a = ops.grouped_gemm(offsets, jagged_a, weight_a, total_rows=R, row_index=index, index_div=K, bias=bias_a)
+        pre_b = ops.grouped_gemm(offsets, jagged_b, weight_b, total_rows=R, row_index=index, index_div=K, bias=bias_b)
+        ctx.save_for_backward(offsets, index, jagged_a, jagged_b, weight_a, weight_b, bias_a, bias_b, pre_a, pre_b)
+        return ops.silu_mul(pre_a, pre_b)
+
+    @staticmethod
+    def backward(ctx, dout):
+        offsets, index, jagged_a, jagged_b, weight_a, weight_b, bias_a, bias_b, pre_a, pre_b = ctx.saved_tensors
+        R, K = index.numel(), index.shape[-1]
+        d_a, d_b = ops.swiglu_bwd(pre_a, pre_b, dout.contiguous())
+        need = ctx.needs_input_grad
+        reverse = _reverse_from_index(index) if need[2] or need[3] else None
+        grads = []
+        for pos, (src, w, bias, d) in enumerate(((jagged_a, weight_a, bias_a, d_a), (jagged_b, weight_b, bias_b, d_b))):
+            d_src = d_w = d_bias = None
+            if need[2 + pos]:
+                d_src = _input_grad([d], [w], offsets, reverse).view_as(src)
+            if need[4 + pos]:
+                operand = _WgradOperand(src, offsets, R, row_index=index.reshape(-1), index_div=K)
+                d_w = operand.weight_grad(d).permute(0, 2, 1)
+            if bias is not None and need[6 + pos]:
+                d_bias = ops.segment_colsum(d, offsets)
+            grads.append((d_src, d_w, d_bias))
+        (da, dwa, dba), (db, dwb, dbb) = grads
+        return None, None, da, db, dwa, dwb, dba, dbb
+
+
+class IndexSelectJaggedBmm3D(torch.autograd.Function):
+    """index_select_jagged_bmm_3D: jagged [L, E, K], expert e reads slice [:, e, :] (backward of
+    kernels/triton/triton_moe.py:1399-1476)."""
+
+    @staticmethod
+    def forward(ctx, offsets, index, jagged, weight, bias):
+        jagged = ops._rows_contiguous(jagged)
+        ctx.save_for_backward(offsets, index, jagged, weight, bias)
+        return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
+                                index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE,
+                                a_expert_stride=jagged.stride(1))
+
+    @staticmethod
+    def backward(ctx, dout):
+        offsets, index, jagged, weight, bias = ctx.saved_tensors
+        L, E, Kin = jagged.shape
+        R, K = index.numel(), index.shape[-1]
+        dout = dout.contiguous()
+        need = ctx.needs_input_grad
+        d_jagged = d_w = d_b = None
+        if need[2] or need[3]:
+            # sorted row r reads slice (token(r), expert(r)) of the input
+            lengths = (offsets[1:] - offsets[:-1]).clamp_min(0)
+            expert = torch.repeat_interleave(torch.arange(E, device=index.device), lengths, output_size=R)
+            cell = torch.div(index.reshape(-1), K, rounding_mode="floor") * E + expert
+        if need[2]:
+            d_rows = ops.grouped_gemm(offsets, dout, weight.permute(0, 2, 1), total_rows=R)
+            # every (token, expert) cell receives the rows routed there, most cells none: summed in
+            # fp32 as the reference does (:1412-1416, 1470); with the distinct experts per token
+            # of a top-k router each cell gets one row at most and the sum has one order
+            acc = torch.zeros((L * E, Kin), dtype=torch.float32, device=dout.device)
+            acc.index_add_(0, cell, d_rows.float())
+            d_jagged = acc.to(jagged.dtype).view(L, E, Kin)
+        if need[3]:
+            src = jagged.contiguous().view(L * E, Kin)
+            d_w = _WgradOperand(src, offsets, R, row_index=cell, index_div=1).weight_grad(dout).permute(0, 2, 1)
+        if bias is not None and need[4]:
+            d_b = ops.segment_colsum(dout, offsets)
+        return None, None, d_jagged, d_w, d_b
+
+
 class MulMergeKAdd(torch.autograd.Function):
     """mul_merge_k_add: weighted deterministic merge."""
 

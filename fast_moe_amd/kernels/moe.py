@@ -111,7 +111,8 @@ def index_select_jagged_bmm_3D(
     require_hip_kernel(kernel, "index_select_jagged_bmm_3D")
     assert index.ndim == 2 and index.shape[0] == jagged.shape[0]
     assert jagged.ndim == 3 and jagged.shape[1] == weight.shape[0]
-    ops._forward_only("index_select_jagged_bmm_3D", jagged, weight, bias)
+    if _ag.needs_grad(jagged, weight, bias):
+        return _ag.IndexSelectJaggedBmm3D.apply(offsets, index, jagged, weight, bias)
     jagged = ops._rows_contiguous(jagged)
     return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                             index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE,
@@ -163,7 +164,9 @@ def index_select_jagged_gating_bmm(
     if jagged_a is jagged_b:
         return index_select_jagged_bmm_swiglu(max_seq_len, offsets, index, jagged_a, weight_a, bias_a,
                                               weight_b, bias_b, kernel)
-    ops._forward_only("index_select_jagged_gating_bmm", jagged_a, jagged_b, weight_a, weight_b, bias_a, bias_b)
+    if _ag.needs_grad(jagged_a, jagged_b, weight_a, weight_b, bias_a, bias_b):
+        return _ag.IndexSelectJaggedGatingBmm.apply(offsets, index, jagged_a, jagged_b, weight_a, weight_b,
+                                                    bias_a, bias_b)
     alpha = ops.grouped_gemm(offsets, jagged_a, weight_a, total_rows=index.numel(), row_index=index,
                              index_div=index.shape[-1], bias=bias_a)
     beta = ops.grouped_gemm(offsets, jagged_b, weight_b, total_rows=index.numel(), row_index=index,

@@ -82,6 +82,55 @@ def test_swiglu_backward(L, E, K, Din, H):
         close(g.grad, q.grad, name, rtol=3e-2, atol_frac=1.5e-2)
 
 
+@pytest.mark.parametrize("L,E,K,Din,H,dtype", [
+    (300, 8, 2, 64, 128, BF16),
+    (2048, 8, 2, 256, 256, BF16),        # in-place weight gradient, ring GEMMs
+    (200, 4, 2, 40, 72, torch.float32),
+])
+def test_gating_bmm_two_inputs_backward(L, E, K, Din, H, dtype):
+    """silu(A Wa + ba) * (B Wb + bb) with A is not B: every gradient (kernels/triton/triton_moe.py:2839-2990)."""
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=11)
+    t0 = [randn((L, Din), 1), randn((L, Din), 2), kn_weight(E, Din, H, 3, False, Din ** -0.5),
+          kn_weight(E, Din, H, 4, True, Din ** -0.5), randn((E, H), 5), randn((E, H), 6)]
+    t0 = [t.to(dtype) for t in t0]
+    dout = (randn((L * K, H), 7) * 0.01).to(dtype)
+    ref = [leaf(t, torch.float32) for t in t0]
+    o_moe.index_select_jagged_gating_bmm(r["offsets"], r["index"], *ref).backward(dout.float())
+    got = [leaf(t, device="cuda") for t in t0]
+    ja, jb, wa, wb, ba, bb = got
+    out = moe.index_select_jagged_gating_bmm(0, dev(r["offsets"]), dev(r["index"]), ja, jb, wa, ba, wb, bb)
+    out.backward(dev(dout))
+    tol = dict(rtol=3e-2, atol_frac=1.5e-2) if dtype == BF16 else dict(rtol=1e-4, atol_frac=1e-5)
+    for name, g, q in zip(("d_jagged_a", "d_jagged_b", "d_weight_a", "d_weight_b", "d_bias_a", "d_bias_b"), got, ref):
+        close(g.grad, q.grad, name, **tol)
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,dtype", [
+    (300, 4, 2, 64, 128, BF16),
+    (1500, 6, 3, 128, 256, BF16),
+    (200, 4, 2, 40, 72, torch.float32),
+])
+def test_bmm_3d_backward(L, E, K, Din, Dout, dtype):
+    """jagged [L, E, Din], expert e reads slice [:, e, :]: every gradient, cells no row reads get zero
+    (kernels/triton/triton_moe.py:1399-1476)."""
+    from fast_moe_amd.kernels import moe
+    r = make_routing(L, E, K, seed=13)
+    x0 = randn((L, E, Din), 1).to(dtype)
+    w0 = kn_weight(E, Din, Dout, 2, False, Din ** -0.5).to(dtype)
+    b0 = randn((E, Dout), 3).to(dtype)
+    dout = (randn((L * K, Dout), 4) * 0.01).to(dtype)
+    xr, wr, br = leaf(x0, torch.float32), leaf(w0, torch.float32), leaf(b0, torch.float32)
+    o_moe.index_select_jagged_bmm_3D(r["offsets"], r["index"], xr, wr, br).backward(dout.float())
+    x, w, b = leaf(x0, device="cuda"), leaf(w0, device="cuda"), leaf(b0, device="cuda")
+    out = moe.index_select_jagged_bmm_3D(0, dev(r["offsets"]), dev(r["index"]), x, w, b)
+    out.backward(dev(dout))
+    tol = dict(rtol=3e-2, atol_frac=1.5e-2) if dtype == BF16 else dict(rtol=1e-4, atol_frac=1e-5)
+    for name, g, q in zip(("d_jagged", "d_weight", "d_bias"), (x, w, b), (xr, wr, br)):
+        close(g.grad, q.grad, name, **tol)
+    assert torch.equal(x.grad.cpu() == 0, xr.grad == 0), "untouched cells"
+
+
 @pytest.mark.parametrize("gate_dtype", [BF16, torch.float32])
 def test_mul_merge_k_add_backward(gate_dtype):
     from fast_moe_amd.kernels import moe
