@@ -264,14 +264,27 @@ class MulMergeKAdd(torch.autograd.Function):
 
 
 class SiluJaggedBmmCombine(torch.autograd.Function):
-    """silu_jagged_bmm_combine: (SiLU,) grouped GEMM + bias, weighted merge."""
+    """silu_jagged_bmm_combine: (SiLU,) grouped GEMM + bias, weighted merge.
+
+    With ``fp8_weight`` = (e4m3 weight [E, D_in, D_out] view, scales): the mixed-precision form of
+    silu_jagged_bmm_combine_fp8, forward GEMM on row-quantised e4m3 operands, backward in bf16 on
+    the original tensors; ``recompute`` drops the GEMM output after the forward and computes it
+    again in bf16 for the gate gradient (SiluJaggedBmmFp8MixedGemmCombine and its
+    activation_checkpointing, kernels/triton/triton_moe_fp8.py:1373-1720)."""
 
     @staticmethod
-    def forward(ctx, offsets, jagged, weight, bias, index, reverse_index, gating_scores, gates_index, has_silu):
-        bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
-                                   epilogue=EPI_NONE, a_silu=has_silu)
+    def forward(ctx, offsets, jagged, weight, bias, index, reverse_index, gating_scores, gates_index, has_silu,
+                fp8_weight=None, recompute=False):
+        if fp8_weight is None:
+            bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
+                                       epilogue=EPI_NONE, a_silu=has_silu)
+        else:
+            qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
+            bmm_out = ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=jagged.shape[0], bias=bias,
+                                       a_scale=sa, b_scale=fp8_weight[1], epilogue=EPI_NONE)
         out = ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
-        ctx.save_for_backward(offsets, jagged, weight, bias, index, gating_scores, gates_index, bmm_out)
+        ctx.save_for_backward(offsets, jagged, weight, bias, index, gating_scores, gates_index,
+                              None if recompute else bmm_out)
         ctx.has_silu = has_silu
         ctx.K = reverse_index.shape[1]
         return out
@@ -279,6 +292,9 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         offsets, jagged, weight, bias, index, gating_scores, gates_index, bmm_out = ctx.saved_tensors
+        if bmm_out is None:
+            bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
+                                       epilogue=EPI_NONE, a_silu=ctx.has_silu)
         need = ctx.needs_input_grad
         need_g = gating_scores is not None and need[6]
         dy = dy.to(bmm_out.dtype)
@@ -295,7 +311,7 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
             d_b = ops.segment_colsum(d_bmm, offsets)
         if need_g:
             d_g = d_gate.view(gating_scores.shape).to(gating_scores.dtype)
-        return None, d_jagged, d_w, d_b, None, None, d_g, None, None
+        return None, d_jagged, d_w, d_b, None, None, d_g, None, None, None, None
 
 
 def needs_grad(*tensors: Optional[torch.Tensor]) -> bool:

@@ -16,6 +16,7 @@ from typing import Optional, Tuple
 
 import torch
 
+from .hip import autograd as _ag
 from .hip import ops
 from .hip._lib import EPI_NONE
 from .utils import KernelType, require_hip_kernel
@@ -154,9 +155,11 @@ def silu_jagged_bmm_combine_fp8(
     require_hip_kernel(kernel, "silu_jagged_bmm_combine_fp8")
     L, K = reverse_index.shape
     assert index.shape[0] == L * K == jagged.shape[0]
-    ops._forward_only("silu_jagged_bmm_combine_fp8", jagged, weight, bias, gating_scores)
-    qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
     qw, sw = cached_quantize_expert_weights(weight)
+    if _ag.needs_grad(jagged, weight, bias, gating_scores):   # forward in e4m3, backward in bf16
+        return _ag.SiluJaggedBmmCombine.apply(offsets, jagged, weight, bias, index, reverse_index, gating_scores,
+                                              gates_index, has_silu, (qw, sw), activation_checkpointing)
+    qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
     bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias, a_scale=sa,
                                b_scale=sw, epilogue=EPI_NONE)
     return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
@@ -177,10 +180,12 @@ def index_select_jagged_bmm(
     (kernels/pytorch/moe_fp8.py:98-139).  fp8=False: the bf16 operator."""
     require_hip_kernel(kernel, "index_select_jagged_bmm")
     assert index.ndim == 2 and index.shape[0] == jagged.shape[0]
-    ops._forward_only("index_select_jagged_bmm", jagged, weight, bias)
     if not fp8:
+        if _ag.needs_grad(jagged, weight, bias):
+            return _ag.IndexSelectJaggedBmm.apply(offsets, index, jagged, weight, bias, None, None)
         return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                                 index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
+    ops._forward_only("index_select_jagged_bmm(fp8=True)", jagged, weight, bias)
     assert jagged.dtype == weight.dtype and (bias is None or jagged.dtype == bias.dtype)
     qa, sa = ops.quant_rows_fp8(jagged)
     qw, sw = cached_quantize_expert_weights(weight)

@@ -174,6 +174,45 @@ def test_silu_jagged_bmm_combine_backward(has_silu):
         close(g.grad, q.grad, name, rtol=3e-2, atol_frac=1.5e-2)
 
 
+@pytest.mark.parametrize("recompute", [False, True])
+def test_silu_jagged_bmm_combine_fp8_trains_in_bf16(recompute):
+    """Forward on e4m3 operands, backward in bf16 on the original tensors
+    (SiluJaggedBmmFp8MixedGemmCombine, kernels/triton/triton_moe_fp8.py:1373-1720): the gradients
+    that do not see the forward GEMM's output meet the bf16 bar; the gate gradient, a dot product
+    with that output, meets it when the output is recomputed in bf16 (activation_checkpointing)
+    and an e4m3 bar otherwise."""
+    from fast_moe_amd.kernels import moe, moe_fp8
+    T, E, K, H, O = 512, 8, 2, 128, 256
+    r = make_routing(T, E, K, seed=13)
+    j0 = randn((T * K, H), 1)
+    w0 = kn_weight(E, H, O, 2, False, H ** -0.5)
+    b0 = randn((E, O), 3)
+    g0 = torch.rand((T, K), generator=torch.Generator().manual_seed(4)).to(BF16)
+    dy = randn((T, O), 5) * 0.01
+    ref = [leaf(t, torch.float32) for t in (j0, w0, b0, g0)]
+    o_moe.silu_jagged_bmm_combine(r["offsets"], ref[0], ref[1], ref[2], r["token_index"], K, ref[3],
+                                  r["gate_index"], True).backward(dy.float())
+    got = [leaf(t, device="cuda") for t in (j0, w0, b0, g0)]
+    args = (dev(r["offsets"]), got[0], got[1], got[2], dev(r["token_index"]), dev(r["reverse_index"]), got[3],
+            dev(r["gate_index"]))
+    out = moe_fp8.silu_jagged_bmm_combine_fp8(0, *args, activation_checkpointing=recompute)
+    with torch.no_grad():       # the forward value is the fp8 operator's own
+        assert torch.equal(out, moe_fp8.silu_jagged_bmm_combine_fp8(0, *args))
+    out.backward(dev(dy))
+    for name, g, q in zip(("d_jagged", "d_weight", "d_bias"), got, ref):
+        close(g.grad, q.grad, name, rtol=3e-2, atol_frac=1.5e-2)
+    loose = {} if recompute else dict(rtol=1e-1, atol_frac=5e-2)
+    close(got[3].grad, ref[3].grad, "d_gates", **(loose or dict(rtol=3e-2, atol_frac=1.5e-2)))
+    # and the bf16 entry point of the fp8 module trains as the bf16 operator does
+    x = leaf(randn((T, H), 6), device="cuda")
+    w = leaf(w0, device="cuda")
+    y = moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, None, fp8=False)
+    y.sum().backward()
+    x2, w2 = leaf(x, device="cuda"), leaf(w, device="cuda")
+    moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x2, w2, None).sum().backward()
+    assert torch.equal(x.grad, x2.grad) and torch.equal(w.grad, w2.grad)
+
+
 def test_layer_backward_matches_oracle():
     """FastMoELayer under grad mode: every parameter and the input receive the oracle's gradient."""
     from fast_moe_amd import FastMoELayer
