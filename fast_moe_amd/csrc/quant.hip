@@ -55,6 +55,33 @@ __device__ __forceinline__ float finish_amax(float m, bool nan) {
     return m;
 }
 
+// eight bf16 values times the row's scale -> eight e4m3 codes.  Rows without NaN / inf take the
+// hardware conversion; a row that holds one goes through the software encoder, which keeps the
+// reference's non-saturating codes.
+__device__ __forceinline__ u32x2 encode8(const u32x4& v, float s, bool special) {
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f[2 * j] = bf16_bits_to_f32(v[j] & 0xffffu) * s;
+        f[2 * j + 1] = __uint_as_float(v[j] & 0xffff0000u) * s;
+    }
+    u32x2 o;
+    if (!special) {
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
+        o[0] = (uint32_t)w0;
+        o[1] = (uint32_t)w1;
+    } else {
+        o[0] = e4m3fn_encode(f[0]) | (e4m3fn_encode(f[1]) << 8) | (e4m3fn_encode(f[2]) << 16) |
+               (e4m3fn_encode(f[3]) << 24);
+        o[1] = e4m3fn_encode(f[4]) | (e4m3fn_encode(f[5]) << 8) | (e4m3fn_encode(f[6]) << 16) |
+               (e4m3fn_encode(f[7]) << 24);
+    }
+    return o;
+}
+
 // ---- fast path: bf16, contiguous columns, cols % 8 == 0, <= CH*512 columns
 template <int CH, bool SILU>
 __global__ __launch_bounds__(256) void quant_rows_bf16_wave(
@@ -100,28 +127,61 @@ __global__ __launch_bounds__(256) void quant_rows_bf16_wave(
     for (int i = 0; i < CH; ++i) {
         const int c = lane + kWave * i;
         if (c >= chunks) continue;
-        float f[8];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            f[2 * j] = bf16_bits_to_f32(v[i][j] & 0xffffu) * s;
-            f[2 * j + 1] = __uint_as_float(v[i][j] & 0xffff0000u) * s;
-        }
-        u32x2 o;
-        if (!special) {
-            int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
-            w0 = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], w0, true);
-            int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
-            w1 = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], w1, true);
-            o[0] = (uint32_t)w0;
-            o[1] = (uint32_t)w1;
-        } else {
-            o[0] = e4m3fn_encode(f[0]) | (e4m3fn_encode(f[1]) << 8) | (e4m3fn_encode(f[2]) << 16) |
-                   (e4m3fn_encode(f[3]) << 24);
-            o[1] = e4m3fn_encode(f[4]) | (e4m3fn_encode(f[5]) << 8) | (e4m3fn_encode(f[6]) << 16) |
-                   (e4m3fn_encode(f[7]) << 24);
-        }
+        const u32x2 o = encode8(v[i], s, special);
         *reinterpret_cast<u32x2*>(dst + (int64_t)c * 8) = o;
     }
+}
+
+// ---- long rows (more columns than a wave holds in registers): one block per row, two passes
+// with 16-byte loads; the second pass finds most of the row in L2.  The transposed operands of
+// the fp8 weight gradient are a few thousand rows of 10^5 columns.
+template <bool SILU>
+__global__ __launch_bounds__(256) void quant_rows_bf16_block(
+    const uint16_t* __restrict__ a, int64_t rows, int64_t cols, int64_t a_sb, int64_t a_sr,
+    uint8_t* __restrict__ q, int64_t q_sb, int64_t q_sr, float* __restrict__ scale, int store_reciprocal) {
+    __shared__ float s_max[4];
+    __shared__ int s_nan[4];
+    const int64_t row = blockIdx.x;
+    const int64_t b = row / rows, r = row - b * rows;
+    const uint16_t* src = a + b * a_sb + r * a_sr;
+    uint8_t* dst = q + b * q_sb + r * q_sr;
+    const int64_t chunks = cols >> 3;
+    auto load = [&](int64_t c) {
+        u32x4 v = *reinterpret_cast<const u32x4*>(src + c * 8);
+        if (SILU) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float lo = round_bf16(silu_f32(bf16_bits_to_f32(v[j] & 0xffffu)));
+                const float hi = round_bf16(silu_f32(__uint_as_float(v[j] & 0xffff0000u)));
+                v[j] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
+            }
+        }
+        return v;
+    };
+    float m = 0.0f;
+    bool nan = false;
+    for (int64_t c = threadIdx.x; c < chunks; c += 256) {
+        const u32x4 v = load(c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            m = amax_update(m, bf16_bits_to_f32(v[j] & 0xffffu), nan);
+            m = amax_update(m, __uint_as_float(v[j] & 0xffff0000u), nan);
+        }
+    }
+    m = wave_max(m);
+    const bool any_nan = __ballot(nan) != 0ull;
+    if (lane_id() == 0) {
+        s_max[threadIdx.x / kWave] = m;
+        s_nan[threadIdx.x / kWave] = any_nan;
+    }
+    __syncthreads();
+    m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    if (s_nan[0] | s_nan[1] | s_nan[2] | s_nan[3]) m = __uint_as_float(0x7fc00000u);
+    const float s = scale_from_amax<true>(m);
+    if (threadIdx.x == 0) scale[row] = store_reciprocal ? 1.0f / s : s;
+    const bool special = !(m <= 3.4028234664e38f);
+    for (int64_t c = threadIdx.x; c < chunks; c += 256)
+        *reinterpret_cast<u32x2*>(dst + c * 8) = encode8(load(c), s, special);
 }
 
 template <typename T>
@@ -253,6 +313,18 @@ extern "C" int fmoe_quant_rows_e4m3(const void* a, int a_dtype, int64_t batch, i
         else if (ch <= 12) FMOE_FAST(12);
         else FMOE_FAST(16);
 #undef FMOE_FAST
+        return check_launch("fmoe_quant_rows_e4m3");
+    }
+    const bool long_rows = a_dtype == FMOE_BF16 && a_sc == 1 && q_sc == 1 && (cols % 8) == 0 && aligned16(a) &&
+                           (a_sb % 8) == 0 && (a_sr % 8) == 0 && (reinterpret_cast<uintptr_t>(q) & 7u) == 0 &&
+                           (q_sb % 8) == 0 && (q_sr % 8) == 0 && total < ((int64_t)1 << 31);
+    if (long_rows) {
+        if (apply_silu)
+            quant_rows_bf16_block<true><<<(unsigned)total, 256, 0, stream>>>((const uint16_t*)a, rows, cols, a_sb, a_sr,
+                                                                             q, q_sb, q_sr, scale, store_reciprocal);
+        else
+            quant_rows_bf16_block<false><<<(unsigned)total, 256, 0, stream>>>((const uint16_t*)a, rows, cols, a_sb, a_sr,
+                                                                              q, q_sb, q_sr, scale, store_reciprocal);
         return check_launch("fmoe_quant_rows_e4m3");
     }
     const bool lane_per_row = a_sc != 1 && a_sr == 1 && rows >= 16;

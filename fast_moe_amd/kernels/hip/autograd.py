@@ -168,6 +168,65 @@ class IndexSelectJaggedBmm(torch.autograd.Function):
         return None, None, d_jagged, d_w, d_b, d_wp, d_bp
 
 
+class IndexSelectJaggedBmmFp8(torch.autograd.Function):
+    """index_select_jagged_bmm(fp8=True): forward and both backward GEMMs on e4m3 operands
+    (kernels/triton/triton_moe_fp8.py:1114-1340).
+
+    Backward, as the reference quantises: d_out per row and the weight per (expert, input row)
+    along the output dimension for the input gradient; the gathered inputs and d_out per
+    COLUMN for the weight gradient.  The column scales are taken over the routed rows in expert
+    order, which hold every token at least once, so they are the reference's scales over all
+    tokens.  The input gradient's rows are rounded to bf16 before the K rows of a token are
+    summed (the reference sums them in fp32)."""
+
+    @staticmethod
+    def forward(ctx, offsets, index, jagged, weight, bias, fp8_weight):
+        qa, sa = ops.quant_rows_fp8(jagged)
+        ctx.save_for_backward(offsets, index, jagged, weight, bias)
+        return ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=index.numel(), row_index=index,
+                                index_div=index.shape[-1], bias=bias, a_scale=sa, b_scale=fp8_weight[1],
+                                epilogue=EPI_NONE)
+
+    @staticmethod
+    def backward(ctx, dout):
+        offsets, index, jagged, weight, bias = ctx.saved_tensors
+        E, Kin, N = weight.shape
+        R, K = index.numel(), index.shape[-1]
+        dout = dout.contiguous()
+        need = ctx.needs_input_grad
+        d_jagged = d_w = d_b = None
+        if need[2]:
+            qd, sd = ops.quant_rows_fp8(dout)                           # [R, N], [R]
+            w_rows = weight
+            if weight.stride(2) != 1 and weight.stride(1) == 1:         # rows along N strided: one transposing copy
+                w_rows = ops.to_k_contiguous(weight.permute(0, 2, 1)).permute(0, 2, 1)
+            qw, sw = ops.quant_rows_fp8(w_rows)                         # [E, Kin, N], [E, Kin]
+            d_rows = ops.grouped_gemm(offsets, qd, qw.permute(0, 2, 1), total_rows=R, a_scale=sd, b_scale=sw)
+            d_jagged = ops.combine(d_rows, _reverse_from_index(index)).view_as(jagged)
+        if need[3]:
+            pad_offsets, bound = _pad_layout(offsets, R)
+            a_t = ops.jagged_transpose(jagged, offsets, pad_offsets, bound, index.reshape(-1), K)   # [Kin, bound]
+            d_t = ops.jagged_transpose(dout, offsets, pad_offsets, bound)                          # [N, bound]
+            qa, sa = ops.quant_rows_fp8(a_t)                            # scales [Kin]
+            qt, st = ops.quant_rows_fp8(d_t)                            # scales [N]
+            # the gradient in the parameter's own memory order: [E, N, Kin] rows for K-contiguous storage
+            by_n = weight.stride(1) == 1 and weight.stride(2) != 1
+            (q_l, s_l, M), (q_r, s_r, C) = ((qt, st, N), (qa, sa, Kin)) if by_n else ((qa, sa, Kin), (qt, st, N))
+            dev = dout.device
+            seg = torch.arange(E + 1, device=dev, dtype=torch.int64) * M
+            rows = torch.arange(E * M, device=dev, dtype=torch.int64) % M
+            b = q_r.t().unsqueeze(0).expand(E, bound, C)                # B[e, r, c] = q_r[c, r]
+            d_w = ops.grouped_gemm(seg, q_l, b, total_rows=E * M, row_index=rows, index_div=1,
+                                   a_scale=s_l, b_scale=s_r.unsqueeze(0).expand(E, C).contiguous(),
+                                   k_window=pad_offsets, k_window_multiple=_WINDOW_MULTIPLE)
+            d_w = d_w.view(E, M, C).to(weight.dtype)
+            if by_n:
+                d_w = d_w.permute(0, 2, 1)
+        if bias is not None and need[4]:
+            d_b = ops.segment_colsum(dout, offsets)
+        return None, None, d_jagged, d_w, d_b, None
+
+
 class IndexSelectJaggedGatingBmm(torch.autograd.Function):
     """index_select_jagged_gating_bmm with two different inputs: silu(A Wa + ba) * (B Wb + bb)
     (backward of kernels/triton/triton_moe.py:2839-2990)."""

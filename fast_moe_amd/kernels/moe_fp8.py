@@ -185,10 +185,11 @@ def index_select_jagged_bmm(
             return _ag.IndexSelectJaggedBmm.apply(offsets, index, jagged, weight, bias, None, None)
         return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                                 index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
-    ops._forward_only("index_select_jagged_bmm(fp8=True)", jagged, weight, bias)
     assert jagged.dtype == weight.dtype and (bias is None or jagged.dtype == bias.dtype)
-    qa, sa = ops.quant_rows_fp8(jagged)
     qw, sw = cached_quantize_expert_weights(weight)
+    if _ag.needs_grad(jagged, weight, bias):
+        return _ag.IndexSelectJaggedBmmFp8.apply(offsets, index, jagged, weight, bias, (qw, sw))
+    qa, sa = ops.quant_rows_fp8(jagged)
     return ops.grouped_gemm(offsets, qa, qw, total_rows=index.numel(), row_index=index,
                             index_div=index.shape[-1], bias=bias, a_scale=sa, b_scale=sw,
                             epilogue=EPI_NONE)

@@ -78,6 +78,54 @@ def index_select_jagged_bmm_fp8(offsets, index, jagged, weight, bias):
     return torch.cat(fp8_linear_per_expert(q_rows, s_rows, q_w, s_w, bias, jagged.dtype), dim=0)
 
 
+def index_select_jagged_bmm_fp8_backward(offsets, index, jagged, weight, bias, d_out):
+    """Backward of the fp8 gather-GEMM as the Triton operator runs it
+    (kernels/triton/triton_moe_fp8.py:1201-1340): every GEMM operand re-quantised to e4m3,
+
+    * d_jagged: d_out quantised per row, weight [E, K, N] per (e, k) row along N; the products
+      are dequantised with the two reciprocal scales (:971-979), land at their [L, A] position
+      in fp32 and are summed over A, then cast (:1244-1249, 1337);
+    * d_weight: jagged and d_out quantised per COLUMN over all their rows
+      (transpose_rowwise_quant, :1281-1286), contracted over the rows of each expert, the
+      left operand gathered by token (:1075-1087), dequantised the same way (:1094-1103);
+    * d_bias: plain per-expert column sums of d_out (:1320-1335).
+
+    Parity pinned by tests/test_oracle_moe.py: on inputs whose quantisation is lossless the three
+    results equal torch autograd through the unquantised operator.
+    Returns (d_jagged [L, K], d_weight [E, K, N], d_bias [E, N] or None)."""
+    L, A = index.shape
+    E, K, N = weight.shape
+    flat = index.reshape(-1)
+    token = flat // A
+    sizes = _sizes(offsets)
+    bounds = [(int(offsets[e]), int(offsets[e + 1])) for e in range(E)]
+
+    qd_c, s_d = rowwise_quant_fp8(d_out)                    # [R, N], [R]
+    qw_c, s_w = rowwise_quant_fp8(weight)                   # [E, K, N], [E, K]
+    qd, qw = dequant(qd_c), dequant(qw_c)
+    expanded = torch.zeros((L * A, K), dtype=torch.float32)
+    for e, (lo, hi) in enumerate(bounds):
+        acc = qd[lo:hi] @ qw[e].T                           # [m_e, K]
+        acc = (acc * (1.0 / s_d[lo:hi])[:, None]) * (1.0 / s_w[e])[None, :]
+        expanded[flat[lo:hi]] = acc
+    d_jagged = expanded.view(L, A, K).sum(dim=1).to(jagged.dtype)
+
+    qjt_c, s_j = (torch.from_numpy(t) for t in _fp8.transpose_rowwise_quant_fp8(
+        jagged.contiguous().float().numpy(), _dtype_name(jagged)))      # [K, L], [K]
+    qdt_c, s_t = (torch.from_numpy(t) for t in _fp8.transpose_rowwise_quant_fp8(
+        d_out.contiguous().float().numpy(), _dtype_name(d_out)))        # [N, R], [N]
+    qjt, qdt = dequant(qjt_c), dequant(qdt_c)
+    d_weight = torch.zeros((E, K, N), dtype=weight.dtype)
+    for e, (lo, hi) in enumerate(bounds):
+        if hi > lo:
+            acc = qjt[:, token[lo:hi]] @ qdt[:, lo:hi].T    # [K, N]
+            d_weight[e] = ((acc * (1.0 / s_j)[:, None]) * (1.0 / s_t)[None, :]).to(weight.dtype)
+    d_bias = None
+    if bias is not None:
+        d_bias = torch.stack([d_out[lo:hi].float().sum(dim=0) for lo, hi in bounds]).to(bias.dtype)
+    return d_jagged, d_weight, d_bias
+
+
 def swiglu_moe_fp8(offsets, index, jagged, w_gate, b_gate, w_up, b_up, w_down, b_down,
                    token_index, k, gates=None, gates_index=None):
     """The fp8 SwiGLU MoE forward as a composition of the emulated fp8 GEMM:

@@ -244,10 +244,40 @@ def test_layer_backward_matches_oracle():
 def test_forward_only_operators_still_refuse_grad():
     from fast_moe_amd.kernels import moe_fp8
     r = make_routing(64, 4, 2, seed=1)
-    x = randn((64, 32), 1).cuda().requires_grad_(True)
+    x = randn((64 * 2, 32), 1).cuda().requires_grad_(True)
     w = randn((4, 32, 32), 2).cuda()
-    with pytest.raises(RuntimeError):
-        moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, None, fp8=True)
+    with pytest.raises(RuntimeError):       # the reference's SiluJaggedBmmFp8 has no backward either
+        moe_fp8.silu_jagged_bmm_fp8(dev(r["offsets"]), 0, x, w, randn((4, 32), 3).cuda())
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,contiguous,with_bias", [
+    (300, 4, 2, 64, 128, True, True),
+    (1200, 8, 2, 256, 384, False, False),
+    (257, 5, 3, 48, 80, True, True),        # short and empty experts, narrow matrices
+])
+def test_index_select_jagged_bmm_fp8_backward(L, E, K, Din, Dout, contiguous, with_bias):
+    """index_select_jagged_bmm(fp8=True) under grad: both backward GEMMs on re-quantised e4m3
+    operands as in kernels/triton/triton_moe_fp8.py:1201-1340, against the oracle's restatement
+    (same quantised operands, fp32 sums; here the input-gradient rows are rounded to bf16 once
+    more before they are summed, hence its wider bar)."""
+    from fast_moe_amd.kernels import moe_fp8
+    from oracle import moe_fp8 as o_fp8
+    r = make_routing(L, E, K, seed=L)
+    x0 = randn((L, Din), 1).to(BF16)
+    w0 = kn_weight(E, Din, Dout, 2, contiguous, Din ** -0.5).to(BF16)
+    b0 = randn((E, Dout), 3).to(BF16) if with_bias else None
+    dout = (randn((L * K, Dout), 4) * 0.01).to(BF16)
+    ref_dx, ref_dw, ref_db = o_fp8.index_select_jagged_bmm_fp8_backward(r["offsets"], r["index"], x0, w0, b0, dout)
+    x, w = leaf(x0, device="cuda"), leaf(w0, device="cuda")
+    b = leaf(b0, device="cuda") if with_bias else None
+    out = moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, b, fp8=True)
+    with torch.no_grad():
+        assert torch.equal(out, moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x, w, b, fp8=True))
+    out.backward(dev(dout))
+    close(w.grad, ref_dw, "d_weight", rtol=1e-2, atol_frac=1e-3)
+    close(x.grad, ref_dx, "d_jagged", rtol=2e-2, atol_frac=4e-3)
+    if with_bias:
+        close(b.grad, ref_db, "d_bias", rtol=1e-2, atol_frac=4e-3)
 
 
 @pytest.mark.parametrize("R,C,E,gather,silu,dtype", [

@@ -45,7 +45,7 @@ def test_reference_shapes(shape, transpose, contiguous, dtype):
 
 
 @pytest.mark.parametrize("rows,cols", [(64, 8), (100, 512), (257, 1408), (300, 2048), (64, 4096), (33, 6000),
-                                       (16, 8192), (5, 8200), (9, 20000)])
+                                       (16, 8192), (5, 8200), (9, 20000), (7, 140032), (3, 9001)])
 def test_wave_per_row_path_and_beyond(rows, cols):
     g = torch.Generator().manual_seed(rows + cols)
     a = (torch.randn(rows, cols, generator=g) * torch.exp(torch.randn(rows, 1, generator=g) * 4)).to(torch.bfloat16)
@@ -88,6 +88,24 @@ def test_special_rows():
     wide[2, 7] = float("nan")
     wide[3] = torch.linspace(-5, 5, 512)
     check_quant(wide.to(torch.bfloat16), both_nan_ok=True)
+
+
+def test_long_rows_special_values_and_silu():
+    """Rows longer than a wave keeps in registers (one block per row, two passes)."""
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(6, 16384, generator=g)
+    a[1, 9000] = float("inf")
+    a[2, 16383] = float("nan")
+    a[3] = 0
+    a[4, 5] = -3.0e38
+    check_quant(a.to(torch.bfloat16), both_nan_ok=True)
+    from fast_moe_amd.kernels.hip import ops
+    from oracle import fp8 as o_fp8
+    x = torch.randn(5, 12288, generator=g).to(torch.bfloat16)
+    q, sc = ops.quant_rows_fp8(x.cuda(), apply_silu=True)
+    ref_q, ref_s = o_fp8.silu_rowwise_quant_fp8(x.float().numpy(), "bf16")
+    assert np.array_equal(q.cpu().view(torch.uint8).numpy(), ref_q)
+    assert np.array_equal(sc.cpu().numpy(), ref_s)
 
 
 def test_fp32_scale_near_power_of_two_follows_reference_formula():

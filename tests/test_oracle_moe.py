@@ -187,6 +187,54 @@ def test_fp8_gemm_agrees_with_dequantised_fp32_oracle():
     torch.testing.assert_close(out.float(), raw, atol=4e-1, rtol=1e-1)
 
 
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_fp8_backward_is_exact_where_quantisation_is_lossless(with_bias):
+    """Integers up to 7 (three significant bits) times a power of two survive e4m3 with the
+    power-of-two scales unchanged, so the fp8 backward must give torch autograd's gradients of
+    the unquantised operator exactly: a wrong gather, a transposed operand, a missing scale or
+    a wrong axis for a scale would each show."""
+    g = torch.Generator().manual_seed(5)
+    L, E, K, Din, Dout = 48, 4, 2, 24, 16
+    _, index, offsets = make_routing(L, E, K, 5)
+
+    def ints(*shape, step):
+        t = torch.randint(-7, 8, shape, generator=g).float() * step
+        t.view(-1, shape[-1])[:, 0] = 7 * step          # every row (and column block) reaches the same amax
+        return t
+    x = ints(L, Din, step=2.0 ** -3)
+    x[0, :] = 7 * 2.0 ** -3                              # ... and every column of x
+    w = ints(E, Din, Dout, step=2.0 ** -5)
+    d_out = ints(L * K, Dout, step=2.0 ** -6)
+    d_out[0, :] = 7 * 2.0 ** -6
+    b = torch.zeros(E, Dout) if with_bias else None
+    xr, wr = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    br = b.clone().requires_grad_(True) if with_bias else None
+    moe_fp8.index_select_jagged_bmm_raw(offsets, index, xr, wr, br).backward(d_out)
+    dx, dw, db = moe_fp8.index_select_jagged_bmm_fp8_backward(offsets, index, x, w, b, d_out)
+    assert torch.equal(dx, xr.grad)
+    assert torch.equal(dw, wr.grad)
+    if with_bias:
+        assert torch.equal(db, br.grad)
+    else:
+        assert db is None
+
+
+def test_fp8_backward_tracks_the_unquantised_gradients():
+    g = torch.Generator().manual_seed(9)
+    L, E, K, Din, Dout = 96, 4, 2, 64, 32
+    _, index, offsets = make_routing(L, E, K, 9)
+    x = torch.empty(L, Din).uniform_(-1, 1, generator=g).to(torch.bfloat16)
+    w = torch.empty(E, Din, Dout).uniform_(-1, 1, generator=g).to(torch.bfloat16)
+    d_out = torch.empty(L * K, Dout).uniform_(-1, 1, generator=g).to(torch.bfloat16)
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    moe_fp8.index_select_jagged_bmm_raw(offsets, index, xr, wr, None).backward(d_out.float())
+    dx, dw, _ = moe_fp8.index_select_jagged_bmm_fp8_backward(offsets, index, x, w, None, d_out)
+    assert dx.dtype == torch.bfloat16 and dw.dtype == torch.bfloat16
+    for got, ref in ((dx, xr.grad), (dw, wr.grad)):
+        err = (got.float() - ref).abs().max() / ref.abs().max()
+        assert err < 0.06, err
+
+
 def test_fp8_swiglu_chain_runs_and_tracks_bf16_chain():
     g = torch.Generator().manual_seed(9)
     L, E, K, D, H = 48, 8, 2, 64, 32
