@@ -3,7 +3,8 @@
 // Fast path (contiguous bf16 rows, cols % 8 == 0): one wavefront per row, the
 // row is read once with 16-byte loads and held in registers, so the traffic is
 // the algorithmic 2 B in + 1 B out per element (+4 B scale per row).
-// Generic paths cover any strides, column counts and fp32 inputs.
+// Rows too long for that (more than 8192 columns) get one block each and two
+// passes.  Generic paths cover any strides, column counts and fp32 inputs.
 #include "common.h"
 
 namespace fmoe {
