@@ -29,6 +29,10 @@ How each function is pinned (no function here is "parity unpinned"):
                                          run-every-expert einsum as an end-to-end check
 * ``moe.mul_merge_k_add``                pure-Python double loop on tiny inputs
 * ``moe_fp8.index_select_jagged_bmm_fp8``  dequantise-then-fp32-oracle agreement
+* ``moe_fp8.index_select_jagged_bmm_fp8_backward``  inputs whose quantisation is
+                                         lossless (small integers times powers of two):
+                                         must equal torch autograd through the
+                                         unquantised operator exactly
 * ``layer.moe_layer_forward``            dense every-expert MoE (the construction of
                                          modules/tests/test_moe_parity.py:72-106)
 """
