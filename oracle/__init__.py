@@ -35,4 +35,7 @@ How each function is pinned (no function here is "parity unpinned"):
                                          unquantised operator exactly
 * ``layer.moe_layer_forward``            dense every-expert MoE (the construction of
                                          modules/tests/test_moe_parity.py:72-106)
+* ``mrn.*`` (SGMoE layer)                the dense-dispatch layer against the
+                                         operator-level oracle on the same routing, the
+                                         comparison kernels/tests/mrn_test.py makes
 """
