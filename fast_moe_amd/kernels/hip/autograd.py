@@ -71,8 +71,7 @@ class _WgradOperand:
                 self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
                 torch.ops.aten.silu.out(a_src, out=self.rows)
             elif not apply_silu:
-                self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
-                torch.index_select(a_src, 0, torch.div(row_index, index_div, rounding_mode="floor"), out=self.rows)
+                self.rows = ops.gather_rows(a_src, torch.div(row_index, index_div, rounding_mode="floor"))
 
     def _transposed(self):
         if self.a_t is None:

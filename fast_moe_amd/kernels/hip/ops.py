@@ -398,8 +398,9 @@ def gemm_plan(d: GemmDesc) -> int:
 
 # ------------------------------------------------------------------ combine
 def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[torch.Tensor] = None,
-            gates_index: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Weighted merge, see fmoe_combine.  value [T*K, D]; reverse_index [T, K]."""
+            gates_index: Optional[torch.Tensor] = None, with_slack: bool = False) -> torch.Tensor:
+    """Weighted merge, see fmoe_combine.  value [T*K, D]; reverse_index [T, K].  ``with_slack``:
+    the output gets SLACK_ROWS readable rows behind it (see empty_rows)."""
     dev = _need_cuda("combine", value, reverse_index, gates, gates_index)
     if value.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"combine: value must be fp32 or bf16, got {value.dtype}")
@@ -426,13 +427,19 @@ def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[to
                 raise ValueError("combine: gates_index must have T*K entries")
     else:
         gates_index = None
-    out = torch.empty((T, D), dtype=out_dtype, device=dev)
+    out = empty_rows(T, D, out_dtype, dev) if with_slack else torch.empty((T, D), dtype=out_dtype, device=dev)
     rc = _lib.load().fmoe_combine(
         value.data_ptr(), _DTYPE_CODE[value.dtype], T, K, D, value.stride(0), reverse_index.data_ptr(),
         _ptr(gates), g_code, g_cols, g_sr, g_sc, _ptr(gates_index), out.data_ptr(), _DTYPE_CODE[out_dtype],
         _stream(value))
     _lib.check(rc, "fmoe_combine")
     return out
+
+
+def gather_rows(src: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    """``src[rows]`` for a 2-D src, as the K = 1 case of the merge kernel (one row per output row,
+    no weights); the result has slack rows behind it."""
+    return combine(src, rows.view(-1, 1), with_slack=True)
 
 
 def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
