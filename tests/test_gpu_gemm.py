@@ -259,13 +259,13 @@ def test_fp8_combine(E, K, Din, Dout, has_silu):
 
 
 def test_forward_only_and_dtype_errors():
-    from fast_moe_amd.kernels import moe
+    from fast_moe_amd.kernels import moe, moe_fp8
     r = make_routing(16, 4, 2)
     x = uniform((16, 32), 1).cuda().requires_grad_()
     w = weights(4, 32, 32, 2).cuda()
-    x3 = uniform((16, 4, 32), 1).cuda().requires_grad_()
-    with pytest.raises(RuntimeError, match="forward-only"):       # no backward for the 3D variant
-        moe.index_select_jagged_bmm_3D(0, dev(r["offsets"]), dev(r["index"]), x3, w, uniform((4, 32), 3).cuda())
+    x2 = uniform((32, 32), 1).cuda().requires_grad_()
+    with pytest.raises(RuntimeError, match="forward-only"):       # no backward for this one, as in the reference
+        moe_fp8.silu_jagged_bmm_fp8(dev(r["offsets"]), 0, x2, w, uniform((4, 32), 3).cuda())
     with pytest.raises(NotImplementedError):
         with torch.no_grad():
             moe.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), x.half(), w.half(), None)
