@@ -203,3 +203,31 @@ def silu_jagged_bmm_combine(
     bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=N, bias=bias, epilogue=EPI_NONE,
                                a_silu=has_silu)
     return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
+
+
+def fused_jagged_bmm_swiglu_combine(
+    offsets: torch.Tensor,
+    index: torch.Tensor,
+    jagged: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    weight_p: torch.Tensor,
+    bias_p: Optional[torch.Tensor],
+    weight_out: torch.Tensor,
+    bias_out: Optional[torch.Tensor],
+    k: int,
+    gates: Optional[torch.Tensor] = None,
+    gates_index: Optional[torch.Tensor] = None,
+    kernel: KernelType = KernelType.HIP,
+) -> torch.Tensor:
+    """kernels/pytorch/moe.py:306-391 (pytorch_fused_jagged_bmm_swiglu_combine): the whole expert
+    block of a SwiGLU MoE, ``merge_k(gates * ((silu(x W + b) * (x Wp + bp)) W_out + b_out))`` ->
+    [L, D].  Three launches (gather + SwiGLU GEMM, down GEMM, merge); differentiable through the
+    two operators it is made of."""
+    require_hip_kernel(kernel, "fused_jagged_bmm_swiglu_combine")
+    assert index.ndim == 2 and index.shape[1] == k, f"{index.shape=}, {k=}"
+    hidden = index_select_jagged_bmm_swiglu(0, offsets, index, jagged, weight, bias, weight_p, bias_p, kernel)
+    token_index = torch.div(index.reshape(-1), k, rounding_mode="floor")
+    reverse_index = _ag._reverse_from_index(index)
+    return silu_jagged_bmm_combine(0, offsets, hidden, weight_out, bias_out, token_index, reverse_index,
+                                   gates, gates_index, has_silu=False, kernel=kernel)

@@ -111,6 +111,10 @@ def test_swiglu_moe_bf16_and_fp8_composition(T, E, K, D, H):
                                                     dev(wg_v), None, dev(wu_v), None)
         y16 = moe.silu_jagged_bmm_combine(0, rg["offsets"], hidden, dev(wd_v), None, rg["token_index"],
                                           rg["reverse_index"], dev(gates), rg["gate_index"], has_silu=False)
+        # the one-call form of the same chain (kernels/pytorch/moe.py:306-391)
+        fused = moe.fused_jagged_bmm_swiglu_combine(rg["offsets"], rg["gate_index"].view(-1, K), dev(x), dev(wg_v), None,
+                                                    dev(wu_v), None, dev(wd_v), None, K, dev(gates), rg["gate_index"])
+        assert torch.equal(fused, y16)
         # fp8: weights quantised once, activations per call
         qg, sg = moe_fp8.quantize_expert_weights(dev(wg_v))
         qu, su = moe_fp8.quantize_expert_weights(dev(wu_v))
@@ -123,6 +127,18 @@ def test_swiglu_moe_bf16_and_fp8_composition(T, E, K, D, H):
         y8 = ops.combine(o8, rg["reverse_index"], dev(gates), rg["gate_index"])
     scale16 = ref16.float().abs().max().item()
     assert_bf16_close(y16, ref16, rtol=1e-2, atol=1e-2 * scale16, what="swiglu bf16")
+    # ... which trains: gradients of the one-call form against autograd through the oracle
+    leaves = [t.detach().float().requires_grad_(True) for t in (x, wg_v, wu_v, wd_v)]
+    dy = torch.randn(T, D, generator=torch.Generator().manual_seed(3)) * 0.01
+    o_moe.fused_jagged_bmm_swiglu_combine(r["offsets"], idx2, leaves[0], leaves[1], None, leaves[2], None, leaves[3],
+                                          None, K, gates.float(), r["gate_index"]).backward(dy)
+    got = [dev(t).detach().requires_grad_(True) for t in (x, wg_v, wu_v, wd_v)]
+    moe.fused_jagged_bmm_swiglu_combine(rg["offsets"], rg["gate_index"].view(-1, K), got[0], got[1], None, got[2], None,
+                                        got[3], None, K, dev(gates), rg["gate_index"]).backward(dev(dy.to(BF16)))
+    for name, g_, q_ in zip(("d_x", "d_w", "d_wp", "d_w_out"), got, leaves):
+        ref_g = q_.grad
+        err = (g_.grad.float().cpu() - ref_g).abs().max().item()
+        assert err <= 3e-2 * ref_g.abs().max().item(), (name, err, ref_g.abs().max().item())
     # fp8 against the oracle's own fp8 path: 3e-2 relative (of the output scale for small entries)
     scale8 = ref8.float().abs().max().item()
     assert_bf16_close(y8, ref8, rtol=3e-2, atol=3e-2 * scale8, what="swiglu fp8")
