@@ -36,3 +36,22 @@ def to_fp32_if_pytorch_kernel(x: torch.Tensor, kernel: KernelType = KernelType.P
     if kernel == KernelType.PYTORCH:
         return x.to(torch.float32)
     return x
+
+
+@torch.fx.wrap
+def fx_torch_zeros_like(t: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """kernels/utils.py:36-38: a leaf for fx tracing."""
+    return torch.zeros_like(t, dtype=dtype)
+
+
+@torch.fx.wrap
+def fx_infer_max_len(lengths: torch.Tensor) -> int:
+    """kernels/utils.py:41-53: the longest expert segment as a host integer (a device-to-host
+    sync).  The HIP operators accept ``max_seq_len`` and ignore it, their tile scheduling reads
+    the offsets on the device, so callers of this package may pass 0 and skip the sync; the
+    helper stays for code that is shared with the reference's back-ends."""
+    longest = int(lengths.max())
+    if not torch.jit.is_scripting() and torch.compiler.is_compiling():
+        torch._check_is_size(longest)      # a size in (0, 10**9) for the compiler's range analysis
+        torch._check(0 < longest < 10 ** 9)
+    return longest

@@ -192,3 +192,16 @@ def test_weight_quant_cache_hits_and_invalidation():
     for _ in range(6):                                    # dead owners are evicted, the table stays bounded
         cache.get(torch.randn(3, 4, 8), quantize)
     assert len(cache._entries) <= 4
+
+
+def test_reference_helper_names_import_without_a_gpu():
+    """Names a caller of the reference imports beside the operators (kernels/utils.py:28-53,
+    utils/configs.py:13-36)."""
+    from fast_moe_amd.kernels.utils import KernelType, fx_infer_max_len, fx_torch_zeros_like, to_fp32_if_pytorch_kernel
+    from fast_moe_amd.utils.configs import MRNOutput, SGConfig
+    assert fx_infer_max_len(torch.tensor([3, 9, 2])) == 9
+    assert fx_torch_zeros_like(torch.ones(2, 3), torch.bfloat16).dtype == torch.bfloat16
+    assert to_fp32_if_pytorch_kernel(torch.ones(1, dtype=torch.bfloat16), KernelType.HIP).dtype == torch.bfloat16
+    cfg = SGConfig(model_d=8, num_experts=4, num_activated_experts=2)
+    assert cfg.loss_coef == 1e-2 and not cfg.enable_noisy_gating
+    assert MRNOutput._fields == ("x", "loss", "load")
