@@ -197,6 +197,7 @@ def test_weight_quant_cache_hits_and_invalidation():
 def test_reference_helper_names_import_without_a_gpu():
     """Names a caller of the reference imports beside the operators (kernels/utils.py:28-53,
     utils/configs.py:13-36)."""
+    import torch
     from fast_moe_amd.kernels.utils import KernelType, fx_infer_max_len, fx_torch_zeros_like, to_fp32_if_pytorch_kernel
     from fast_moe_amd.utils.configs import MRNOutput, SGConfig
     assert fx_infer_max_len(torch.tensor([3, 9, 2])) == 9
