@@ -457,3 +457,71 @@ def test_two_products_in_one_gemm(lens, K1, K2, N):
     wk = w.transpose(1, 2).contiguous().transpose(1, 2)      # k contiguous
     wk2 = w2.transpose(1, 2).contiguous().transpose(1, 2)
     assert ops.grouped_gemm_sum2(offsets.cuda(), a, wk, a2, wk2, total_rows=R) is None
+
+
+def test_full_size_c3_training_step_sampled():
+    """BASELINE's bf16 configuration (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed routing with
+    empty experts) forward + backward through the one-call expert block.  Checked: (1) a sample
+    of token gradients and the weight gradients of the smallest non-empty expert against fp32
+    autograd on just those rows; (2) size-independent: gradients are linear in the incoming
+    gradient (twice the incoming gradient gives exactly twice every gradient, a power of two
+    commutes with every rounding) and experts without rows receive exactly zero."""
+    from fast_moe_amd.kernels import moe
+    from helpers import skewed_topk
+    from oracle import routing as o_routing
+    T, E, K, D, H = 16384, 64, 8, 2048, 1408
+    topk = skewed_topk(T, E, K, seed=11)
+    meta = o_routing.routing_metadata(topk.numpy(), E)
+    lengths = torch.from_numpy(meta["lengths"])
+    offsets = torch.from_numpy(meta["offsets"])
+    gate_index = torch.from_numpy(meta["gate_index"])
+    token_index = gate_index // K
+    g = torch.Generator().manual_seed(0)
+    x0 = torch.randn(T, D, generator=g).to(BF16)
+    wg0 = (torch.randn(E, H, D, generator=g) * D ** -0.5).to(BF16).permute(0, 2, 1)
+    wu0 = (torch.randn(E, H, D, generator=g) * D ** -0.5).to(BF16).permute(0, 2, 1)
+    wd0 = (torch.randn(E, D, H, generator=g) * H ** -0.5).to(BF16).permute(0, 2, 1)
+    gates0 = torch.rand(T, K, generator=g).to(BF16)
+    dy = (torch.randn(T, D, generator=g) * 0.01).to(BF16)
+
+    def step(scale):
+        leaves = [dev(t).detach().requires_grad_(True) for t in (x0, wg0, wu0, wd0)]
+        y = moe.fused_jagged_bmm_swiglu_combine(dev(offsets), dev(gate_index).view(T, K), leaves[0], leaves[1], None,
+                                                leaves[2], None, leaves[3], None, K, dev(gates0), dev(gate_index))
+        y.backward(dev(dy) * scale)
+        return [t.grad for t in leaves]
+
+    grads = step(1.0)
+    twice = step(2.0)
+    for name, a, b in zip(("d_x", "d_wg", "d_wu", "d_wd"), grads, twice):
+        assert torch.equal(a * 2, b), f"{name}: not linear in the incoming gradient"
+    empty = (lengths == 0).nonzero().view(-1)
+    assert empty.numel() >= 2
+    for a in grads[1:]:
+        assert not a[dev(empty)].any()
+    dx, dwg, dwu, dwd = (t.float().cpu() for t in grads)
+    gate_of_row = gates0.reshape(-1)[gate_index].float()          # gates_index = gate_index
+
+    def rows_loss(rows, x_rows, wg, wu, wd):
+        h = torch.nn.functional.silu(x_rows @ wg) * (x_rows @ wu)
+        return ((h @ wd) * dy.float()[token_index[rows]] * gate_of_row[rows][:, None]).sum()
+
+    # weight gradients of the smallest expert that has rows
+    e = int(torch.where(lengths > 0, lengths, lengths.max() + 1).argmin())
+    rows = torch.arange(int(offsets[e]), int(offsets[e + 1]))
+    w = [t[e].float().requires_grad_(True) for t in (wg0, wu0, wd0)]
+    rows_loss(rows, x0.float()[token_index[rows]], *w).backward()
+    for name, got, ref in zip(("d_wg", "d_wu", "d_wd"), (dwg[e], dwu[e], dwd[e]), (t.grad for t in w)):
+        close(got, ref, f"{name}[{e}] ({rows.numel()} rows)", rtol=3e-2, atol_frac=1.5e-2)
+    # input gradients of a few tokens: their K rows, each with its own expert
+    expert_of_row = torch.searchsorted(offsets[1:], torch.arange(T * K), right=True)
+    inv = torch.empty(T * K, dtype=torch.int64)
+    inv[gate_index] = torch.arange(T * K)
+    for t in (0, 4097, T - 1):
+        xt = x0[t].float().requires_grad_(True)
+        total = 0
+        for r in inv[t * K:(t + 1) * K].tolist():
+            ee = int(expert_of_row[r])
+            total = total + rows_loss(torch.tensor([r]), xt[None, :], wg0[ee].float(), wu0[ee].float(), wd0[ee].float())
+        total.backward()
+        close(dx[t], xt.grad, f"d_x[{t}]", rtol=3e-2, atol_frac=2e-2)
