@@ -66,6 +66,7 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     if (two)
         FMOE_REQUIRE(d->b2 && d->k2 >= 1 && d->epilogue == FMOE_EPI_NONE && !d->k_window && !row_indexed,
                      "fmoe_grouped_gemm: a2 needs b2 and k2, and goes with no epilogue and no k_window");
+    if (two) FMOE_REQUIRE(d->k <= (1 << 30) && d->k2 <= (1 << 30), "fmoe_grouped_gemm: k + k2 does not fit 32 bits");
     const int ktot = d->k + (two ? d->k2 : 0);
     if (fp8) {
         FMOE_REQUIRE(d->a_scale && d->b_scale, "fmoe_grouped_gemm: e4m3 operands need a_scale and b_scale");
