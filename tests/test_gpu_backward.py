@@ -525,3 +525,35 @@ def test_full_size_c3_training_step_sampled():
             total = total + rows_loss(torch.tensor([r]), xt[None, :], wg0[ee].float(), wu0[ee].float(), wd0[ee].float())
         total.backward()
         close(dx[t], xt.grad, f"d_x[{t}]", rtol=3e-2, atol_frac=2e-2)
+
+
+@pytest.mark.parametrize("L,E,K,Din,Dout,contiguous,has_bias", [
+    (16, 4, 2, 32, 16, True, True),
+    (32, 8, 4, 64, 32, False, False),
+    (100, 16, 2, 32, 32, False, True),
+    (500, 4, 4, 64, 16, True, False),
+    (500, 16, 4, 64, 32, False, True),
+])
+def test_fp8_gather_gemm_against_the_unquantised_operator(L, E, K, Din, Dout, contiguous, has_bias):
+    """The reference's own fp8 check (kernels/tests/moe_fp8_test.py:296-335, 372-507): the fp8
+    operator against the unquantised one on uniform(-1, 1) inputs, forward and all gradients,
+    atol 4e-1 / rtol 1e-1, over its grid of sizes, weight layouts and bias."""
+    from fast_moe_amd.kernels import moe_fp8
+    from oracle import moe_fp8 as o_fp8
+    from helpers import uniform
+    r = make_routing(L, E, K, seed=L + E)
+    x0, b0 = uniform((L, Din), 1), uniform((E, Dout), 3)
+    w0 = uniform((E, Din, Dout), 2)
+    if not contiguous:
+        w0 = w0.transpose(1, 2).contiguous().transpose(1, 2)
+    dout = (randn((L * K, Dout), 4) * 0.01).to(BF16)
+    ref = [leaf(t, torch.float32) for t in (x0, w0, b0)]
+    out_ref = o_fp8.index_select_jagged_bmm_raw(r["offsets"], r["index"], ref[0], ref[1], ref[2] if has_bias else None)
+    out_ref.backward(dout.float())
+    got = [leaf(t, device="cuda") for t in (x0, w0, b0)]
+    out = moe_fp8.index_select_jagged_bmm(0, dev(r["offsets"]), dev(r["index"]), got[0], got[1],
+                                          got[2] if has_bias else None, fp8=True)
+    torch.testing.assert_close(out.float().cpu(), out_ref.detach(), atol=4e-1, rtol=1e-1)
+    out.backward(dev(dout))
+    for g_, q_ in zip(got[:2 + has_bias], ref):
+        torch.testing.assert_close(g_.grad.float().cpu(), q_.grad, atol=4e-1, rtol=1e-1)
