@@ -540,3 +540,43 @@ def test_ring_kernel_reads_n_contiguous_weights_in_place(L, E, K, Din, Dout, epi
     wide[:, :, 8:8 + Dout] = w
     if epi == "none":
         assert torch.equal(ops.grouped_gemm(off, x, wide[:, :, 8:8 + Dout], **kw), ref)
+
+
+@pytest.mark.parametrize("G", [1, 4, 16])
+@pytest.mark.parametrize("M", [0, 64, 512, 1000000])
+@pytest.mark.parametrize("K,fp8", [(29, False), (256, False), (256, True)])
+def test_reference_grouped_gemm_grid(G, M, K, fp8):
+    """The grid of kernels/tests/grouped_gemm_test.py:28-199: M rows cut at G - 1 random points
+    (empty groups included), N = 256, weights [G * N, K]; bf16 against the fp32 product (atol
+    1e-5, rtol 1.6e-2 there; the absolute term here is scaled to sqrt(K)-sized sums), e4m3
+    against the product of the dequantised operands (2e-2 / 5e-2 and 1.6e-2).  The million-row
+    case is checked on the GPU in fp32, expert by expert."""
+    from fast_moe_amd.kernels.hip import ops
+    N = 256
+    g = torch.Generator().manual_seed(G * 1000 + M % 997 + K)
+    a = torch.randn(M, K, generator=g).to(BF16).cuda()
+    b = torch.randn(G * N, K, generator=g).to(BF16).cuda()
+    cuts = torch.sort(torch.randint(0, max(M, 1), (G - 1,), generator=g)).values if M > 0 else torch.zeros(G - 1, dtype=torch.int64)
+    offsets = torch.cat([torch.zeros(1, dtype=torch.int64), cuts.to(torch.int64), torch.tensor([M])])
+    w = b.view(G, N, K).permute(0, 2, 1)                      # [G, K, N], K contiguous
+    if fp8:
+        qa, sa = ops.quant_rows_fp8(a) if M else (torch.empty((0, K), dtype=ops.FP8_DTYPE, device="cuda"), torch.empty(0, device="cuda"))
+        qb, sb = ops.quant_rows_fp8(b)
+        out = ops.grouped_gemm(offsets.cuda(), qa, qb.view(G, N, K).permute(0, 2, 1), total_rows=M,
+                               a_scale=sa, b_scale=sb.view(G, N))
+    else:
+        out = ops.grouped_gemm(offsets.cuda(), a, w, total_rows=M)
+    assert tuple(out.shape) == (M, N) and out.dtype == BF16
+    if M == 0:
+        return
+    for e in range(G):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if lo == hi:
+            continue
+        if fp8:
+            ref = (qa[lo:hi].float() @ qb.view(G, N, K)[e].float().T) / (sa[lo:hi, None] * sb.view(G, N)[e][None, :])
+            atol = 5e-2 if M > 16384 else 2e-2
+        else:
+            ref = a[lo:hi].float() @ w[e].float()
+            atol = 1e-5 + 4e-3 * K ** 0.5
+        torch.testing.assert_close(out[lo:hi].float(), ref.to(BF16).float(), atol=atol, rtol=1.6e-2)
