@@ -557,3 +557,26 @@ def test_fp8_gather_gemm_against_the_unquantised_operator(L, E, K, Din, Dout, co
     out.backward(dev(dout))
     for g_, q_ in zip(got[:2 + has_bias], ref):
         torch.testing.assert_close(g_.grad.float().cpu(), q_.grad, atol=4e-1, rtol=1e-1)
+
+
+@pytest.mark.parametrize("N", [32768 * 32 * 128, 391336 * 2 * 1024])
+@pytest.mark.parametrize("dtype", [torch.float32, BF16])
+def test_silu_backward_at_the_reference_sizes(N, dtype):
+    """kernels/tests/general_ops_test.py:24-66: SiLU backward on 1.3 * 10^8 and 8 * 10^8 elements
+    against torch autograd with assert_close's default tolerances; and the gated form on the
+    smaller size."""
+    from fast_moe_amd.kernels.hip import ops
+    g = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.empty(N, device="cuda", dtype=dtype).uniform_(-1.0, 1.0, generator=g).requires_grad_()
+    dy = torch.randn(N, device="cuda", dtype=dtype, generator=g) * 0.01
+    torch.nn.functional.silu(x).backward(dy)
+    dx = ops.swiglu_bwd(x.detach().view(-1, 1024), None, dy.view(-1, 1024))[0].view(-1)
+    torch.testing.assert_close(dx, x.grad)
+    if N > 2 ** 28:
+        return
+    x.grad = None
+    u = torch.empty(N, device="cuda", dtype=dtype).uniform_(-1.0, 1.0, generator=g).requires_grad_()
+    (torch.nn.functional.silu(x) * u).backward(dy)
+    dg, du = ops.swiglu_bwd(x.detach().view(-1, 1024), u.detach().view(-1, 1024), dy.view(-1, 1024))
+    torch.testing.assert_close(dg.view(-1), x.grad)
+    torch.testing.assert_close(du.view(-1), u.grad)
