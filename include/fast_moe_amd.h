@@ -50,12 +50,16 @@ enum fmoe_status {
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int fmoe_version(void);
 
-/* Message of the last non-zero return on this thread ("" if none). */
+/* Message of the last non-zero return on this thread ("" if none).  No reference counterpart:
+ * its errors are Python assert / ValueError / NotImplementedError (kernels/moe.py:277-280,
+ * kernels/moe_fp8.py:73-74); the Python layer above this library raises from this message. */
 const char* fmoe_last_error(void);
 
 /* ------------------------------------------------------------------ routing */
 
-/* Bytes of scratch fmoe_route_topk / fmoe_route_from_topk need for (T, E, K). */
+/* Bytes of scratch fmoe_route_topk / fmoe_route_from_topk need for (T, E, K).  No reference
+ * counterpart: its two sorts allocate inside torch (modules/fast_moe_module.py:107-144); here
+ * the caller owns every byte. */
 size_t fmoe_route_workspace_bytes(int64_t T, int E, int K);
 
 /*
@@ -155,8 +159,9 @@ int fmoe_quant_rows_e4m3(const void* a, int a_dtype, int64_t batch, int64_t rows
  *
  * With k_window the contraction range differs per expert: this is the weight
  * gradient of the operators above, dW[e] = A_e^T x dOut_e reduced over the rows of
- * expert e (kernels/triton/triton_moe.py:1793-1976, 4030-4108), computed on the
- * transposed, zero-padded operands fmoe_jagged_transpose writes.
+ * expert e (kernels/triton/triton_moe.py:1793-1976, 4030-4108), computed either on the
+ * transposed, zero-padded operands fmoe_jagged_transpose writes or, with a_stride_k, on the
+ * row-major tensors themselves.
  */
 typedef struct fmoe_gemm_desc {
     int32_t num_experts;    /* E                                                  */
