@@ -433,6 +433,7 @@ def test_weight_gradient_from_rows_in_place(lens):
 @pytest.mark.parametrize("lens,K1,K2,N", [
     ([300, 0, 1000, 128, 77, 515], 256, 256, 256),
     ([4096, 640], 384, 384, 520),
+    ([(37 * i) % 300 + 8 for i in range(100)], 128, 128, 256),      # 100 experts: the wider register tables
 ])
 def test_two_products_in_one_gemm(lens, K1, K2, N):
     """out = a @ b + a2 @ b2 (the SwiGLU input gradient) in one pass: bit-identical to the same
