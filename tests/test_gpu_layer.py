@@ -177,3 +177,34 @@ def test_layer_fp32_matches_oracle(B, S, D, H, O, E, k):
                                             r2["gate_index"]).view(B, S, O)
     assert y.dtype == torch.float32
     torch.testing.assert_close(y.cpu(), ref, atol=1e-4, rtol=1e-4)
+
+
+def test_layer_forward_replays_from_a_captured_graph():
+    """Serving loops replay the forward from a HIP graph: the library neither allocates nor
+    synchronises nor clears memory with memset nodes, so the whole layer (gate, routing, both
+    GEMMs, merge) captures.  Every replay, with eager work and synchronisations in between, must
+    give the eager result of its input bit for bit, routing included (decode-sized and larger)."""
+    from fast_moe_amd.modules.fast_moe_module import FastMoELayer
+    torch.manual_seed(0)
+    D, H, O, E, k = 256, 512, 256, 16, 4
+    layer = FastMoELayer(D, H, O, E).to(BF16).cuda()
+    for B, S in ((1, 8), (4, 300)):
+        static_x = torch.zeros(B, S, D, dtype=BF16, device="cuda")
+        with torch.no_grad():
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):                 # warm-up outside the capture
+                layer(static_x, k)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_y = layer(static_x, k)
+            for seed in range(4):
+                x = randn((B, S, D), 100 + seed).cuda()
+                eager = layer(x, k)                       # eager work between the replays
+                torch.cuda.synchronize()
+                static_x.copy_(x)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(static_y, eager), (B, S, seed)
+        del graph
