@@ -201,9 +201,16 @@ __global__ __launch_bounds__(256) void swiglu_bwd_bf16x8_kernel(const uint16_t* 
                                                                 const uint16_t* __restrict__ u,
                                                                 const uint16_t* __restrict__ dh,
                                                                 uint16_t* __restrict__ dg,
-                                                                uint16_t* __restrict__ du, int64_t n8) {
+                                                                uint16_t* __restrict__ du, int64_t n8,
+                                                                int64_t cols8, int64_t out_stride8) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n8) return;
+    // outputs with a row pitch of their own (out_stride8 chunks per row of cols8 chunks)
+    int64_t o = i;
+    if (out_stride8 != cols8) {
+        const int64_t row = i / cols8;
+        o = row * out_stride8 + (i - row * cols8);
+    }
     const u32x4 vg = reinterpret_cast<const u32x4*>(g)[i];
     const u32x4 vd = reinterpret_cast<const u32x4*>(dh)[i];
     u32x4 vu = {0, 0, 0, 0}, og, ou = {0, 0, 0, 0};
@@ -228,8 +235,8 @@ __global__ __launch_bounds__(256) void swiglu_bwd_bf16x8_kernel(const uint16_t* 
         og[q] = rg;
         ou[q] = ru;
     }
-    reinterpret_cast<u32x4*>(dg)[i] = og;
-    if (GATED) reinterpret_cast<u32x4*>(du)[i] = ou;
+    reinterpret_cast<u32x4*>(dg)[o] = og;
+    if (GATED) reinterpret_cast<u32x4*>(du)[o] = ou;
 }
 
 struct GateArgs {
@@ -357,11 +364,19 @@ extern "C" int fmoe_segment_colsum(const void* src, int dtype, int64_t total_row
 }
 
 extern "C" int fmoe_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* du, int dtype,
-                               int64_t n, fmoe_stream_t stream) {
+                               int64_t n, int64_t cols, int64_t out_stride_row, fmoe_stream_t stream) {
     FMOE_REQUIRE(dtype == FMOE_BF16 || dtype == FMOE_F32, "fmoe_swiglu_bwd: dtype must be bf16 or fp32");
     FMOE_REQUIRE(n >= 0, "fmoe_swiglu_bwd: n < 0");
     if (n == 0) return FMOE_OK;
     FMOE_REQUIRE(g && dh && dg && (!u || du), "fmoe_swiglu_bwd: NULL pointer");
+    const bool pitched = out_stride_row != 0 && out_stride_row != cols;
+    if (pitched)
+        FMOE_REQUIRE(dtype == FMOE_BF16 && cols >= 8 && cols % 8 == 0 && n % cols == 0 && out_stride_row > cols &&
+                         out_stride_row % 8 == 0 && aligned16(g) && aligned16(dh) && aligned16(dg) &&
+                         (!u || (aligned16(u) && aligned16(du))),
+                     "fmoe_swiglu_bwd: outputs with a row pitch need bf16, cols and pitch in multiples of 8, "
+                     "16-byte alignment (cols=%lld pitch=%lld)", (long long)cols, (long long)out_stride_row);
+    const int64_t cols8 = pitched ? cols / 8 : 1, stride8 = pitched ? out_stride_row / 8 : 1;
     const unsigned blocks = (unsigned)((n + 255) / 256);
     FMOE_REQUIRE((n + 255) / 256 < ((int64_t)1 << 31), "fmoe_swiglu_bwd: too many elements");
     hipStream_t s = (hipStream_t)stream;
@@ -369,8 +384,8 @@ extern "C" int fmoe_swiglu_bwd(const void* g, const void* u, const void* dh, voi
         (!u || (aligned16(u) && aligned16(du)))) {
         const int64_t n8 = n / 8;
         const unsigned b8 = (unsigned)((n8 + 255) / 256);
-        if (u) swiglu_bwd_bf16x8_kernel<true><<<b8, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)u, (const uint16_t*)dh, (uint16_t*)dg, (uint16_t*)du, n8);
-        else swiglu_bwd_bf16x8_kernel<false><<<b8, 256, 0, s>>>((const uint16_t*)g, nullptr, (const uint16_t*)dh, (uint16_t*)dg, nullptr, n8);
+        if (u) swiglu_bwd_bf16x8_kernel<true><<<b8, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)u, (const uint16_t*)dh, (uint16_t*)dg, (uint16_t*)du, n8, cols8, stride8);
+        else swiglu_bwd_bf16x8_kernel<false><<<b8, 256, 0, s>>>((const uint16_t*)g, nullptr, (const uint16_t*)dh, (uint16_t*)dg, nullptr, n8, cols8, stride8);
     } else if (dtype == FMOE_BF16) {
         if (u) swiglu_bwd_kernel<uint16_t, true><<<blocks, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)u, (const uint16_t*)dh, (uint16_t*)dg, (uint16_t*)du, n);
         else swiglu_bwd_kernel<uint16_t, false><<<blocks, 256, 0, s>>>((const uint16_t*)g, nullptr, (const uint16_t*)dh, (uint16_t*)dg, nullptr, n);

@@ -79,6 +79,15 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     p.E = d->num_experts;
     p.N = d->n;
     p.K = ktot;
+    p.out2 = (uint16_t*)d->out2;
+    p.out_half = 0;
+    if (d->out2) {
+        FMOE_REQUIRE(row_indexed && d->total_rows % (2 * (int64_t)d->num_experts) == 0 &&
+                         (d->total_rows / (2 * (int64_t)d->num_experts)) % 32 == 0 && aligned16(d->out2),
+                     "fmoe_grouped_gemm: out2 goes with a_stride_k and experts of 2 * h output rows each, h a "
+                     "multiple of 32 (total_rows=%lld E=%d)", (long long)d->total_rows, d->num_experts);
+        p.out_half = d->total_rows / (2 * (int64_t)d->num_experts);
+    }
     p.a2 = (const uint8_t*)d->a2;
     p.k_split = d->k;
     p.index_div = d->index_div;

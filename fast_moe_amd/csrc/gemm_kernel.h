@@ -70,6 +70,8 @@ struct GemmParams {
     uint16_t* aux;                      // SWIGLU: the two pre-activations, or null
     uint16_t* aux2;
     int64_t aux_stride;
+    uint16_t* out2;                     // XTR: rows [out_half, 2 * out_half) of every expert's result go here, or null
+    int64_t out_half;
     const uint8_t* a2;                  // second product a2 * b2 summed into the same output, or null
     int k_split;                        // ... whose contraction covers k in [k_split, K)
 };
@@ -137,7 +139,10 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
 // ALWAYS_VEC: the caller has checked p.vec_store (the ring kernel is only chosen with it), so
 // the element-store path is not even compiled in.  ROWS32: total_rows < 2^31 (the paired ring's
 // condition), so row numbers and row_index values fit 32 bits.
-template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false, bool ROWS32 = false>
+// OUT2: an expert's output rows are split in two halves that go to two tensors (p.out2; the
+// weight gradients of two matrices from one GEMM); a 32-row block lies in one half.
+template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false, bool ROWS32 = false,
+          bool OUT2 = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
                                               int lane) {
@@ -329,7 +334,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         }
                     };
                     const int64_t block_row = row0 + wm * TM + fm * 32;
-                    store(o, p.out + block_row * p.out_stride, p.out_stride);
+                    uint16_t* obase = p.out + block_row * p.out_stride;
+                    if constexpr (OUT2) {
+                        if (p.out2) {       // (scalar arithmetic: everything here is wave-uniform)
+                            const int64_t m = block_row - (int64_t)expert * (2 * p.out_half);
+                            const bool upper = m >= p.out_half;
+                            obase = (upper ? p.out2 : p.out) +
+                                    ((int64_t)expert * p.out_half + (upper ? m - p.out_half : m)) * p.out_stride;
+                        }
+                    }
+                    store(o, obase, p.out_stride);
                     if (HAS_AUX) {
                         store(pg, p.aux + block_row * p.aux_stride, p.aux_stride);
                         store(pu, p.aux2 + block_row * p.aux_stride, p.aux_stride);
@@ -1622,8 +1636,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         cur = nxt;          // valid when another tile follows
         if (EARLY_ROWS) prefetch_next();    // nxt: the tile after that one; its row indices arrive during the epilogue
 
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
-                                                done.rows_valid, wm, wn, lane);
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
+                                                                done.rows_valid, wm, wn, lane);
     }
     wait_vmcnt<0>();    // nothing may still be on its way into this block's LDS when it ends
 }

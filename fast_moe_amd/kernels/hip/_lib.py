@@ -47,7 +47,7 @@ class GemmDesc(ctypes.Structure):
         ("aux2", c_void_p),
         ("aux_stride_row", c_int64),
         ("a_stride_k", c_int64),
-        ("a2", c_void_p), ("k2", c_int32), ("reserved1", c_int32),
+        ("a2", c_void_p), ("k2", c_int32), ("reserved1", c_int32), ("out2", c_void_p),
     ]
 
 
@@ -98,7 +98,8 @@ def load() -> ctypes.CDLL:
     lib.fmoe_segment_colsum.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
                                         c_void_p]
     lib.fmoe_swiglu_bwd.restype = c_int
-    lib.fmoe_swiglu_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_void_p]
+    lib.fmoe_swiglu_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
+                                    c_int64, c_void_p]
     lib.fmoe_combine_bwd.restype = c_int
     lib.fmoe_combine_bwd.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_int64, c_void_p,
                                      c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,

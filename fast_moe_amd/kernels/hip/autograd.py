@@ -80,6 +80,14 @@ class _WgradOperand:
             self.a_t = ops.jagged_transpose(a_src, self.offsets, self.pad_offsets, self.bound, row_index, index_div,
                                             apply_silu)
 
+    def weight_grad_pair(self, both: torch.Tensor):
+        """The weight gradients of two matrices whose row gradients lie side by side in ``both``
+        [rows, 2 N], from one GEMM: ([E, N, K_in], [E, N, K_in]), or None when the operands do not
+        qualify for the in-place kernel."""
+        if self.rows is None:
+            return None
+        return ops.jagged_weight_grad(both, self.rows, self.offsets, halves=True)
+
     def weight_grad(self, dout: torch.Tensor) -> torch.Tensor:
         """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a(r)[k] -> [E, N, K_in]."""
         if self.rows is not None:
@@ -143,10 +151,12 @@ class IndexSelectJaggedBmm(torch.autograd.Function):
         R = index.numel()
         dout = dout.contiguous()
         swiglu = weight_p is not None
-        if swiglu:
-            dg, du = ops.swiglu_bwd(g, u, dout)
+        both = None
+        if swiglu:      # dg | du side by side in one buffer: the GEMMs that need both read one operand
+            dg, du = ops.swiglu_bwd(g, u, dout, joint=True)
             del g, u
             drows, weights = [dg, du], [weight, weight_p]
+            both = ops.joint_rows(dg, du)
         else:
             drows, weights = [dout], [weight]
         need = ctx.needs_input_grad
@@ -156,14 +166,27 @@ class IndexSelectJaggedBmm(torch.autograd.Function):
         operand = None
         if need[3] or (swiglu and need[5]):
             operand = _WgradOperand(jagged, offsets, R, row_index=index.reshape(-1), index_div=K)
-        if need[3]:
-            d_w = operand.weight_grad(drows[0]).permute(0, 2, 1)
-        if bias is not None and need[4]:
-            d_b = ops.segment_colsum(drows[0], offsets)
-        if swiglu and need[5]:
-            d_wp = operand.weight_grad(drows[1]).permute(0, 2, 1)
-        if swiglu and bias_p is not None and need[6]:
-            d_bp = ops.segment_colsum(drows[1], offsets)
+        H = drows[0].shape[1]
+        pair = None
+        if both is not None and need[3] and need[5]:
+            # one GEMM for both weight gradients (2H = 2816 rows per expert fill whole 256-row tiles
+            # where H = 1408 leaves every sixth one half empty), each into its own tensor
+            pair = operand.weight_grad_pair(both)
+        if pair is not None:
+            d_w, d_wp = pair[0].permute(0, 2, 1), pair[1].permute(0, 2, 1)
+        else:
+            if need[3]:
+                d_w = operand.weight_grad(drows[0]).permute(0, 2, 1)
+            if swiglu and need[5]:
+                d_wp = operand.weight_grad(drows[1]).permute(0, 2, 1)
+        if both is not None and bias is not None and bias_p is not None and need[4] and need[6]:
+            d_sum = ops.segment_colsum(both, offsets)
+            d_b, d_bp = d_sum[:, :H], d_sum[:, H:]
+        else:
+            if bias is not None and need[4]:
+                d_b = ops.segment_colsum(drows[0], offsets)
+            if swiglu and bias_p is not None and need[6]:
+                d_bp = ops.segment_colsum(drows[1], offsets)
         return None, None, d_jagged, d_w, d_b, d_wp, d_bp
 
 

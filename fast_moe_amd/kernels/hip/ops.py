@@ -196,11 +196,12 @@ def slack_rows(t: torch.Tensor) -> int:
     return max(0, (have - t.shape[1]) // t.stride(0) + 1 - t.shape[0]) if t.stride(0) > 0 else 0
 
 
-def jagged_weight_grad(dout: torch.Tensor, a_rows: torch.Tensor, offsets: torch.Tensor) -> Optional[torch.Tensor]:
+def jagged_weight_grad(dout: torch.Tensor, a_rows: torch.Tensor, offsets: torch.Tensor, halves: bool = False):
     """dW[e, n, k] = sum over the rows r of expert e of dout[r, n] * a_rows[r, k] -> [E, N, K_in],
     both operands read in place (fmoe_grouped_gemm with a_stride_k).  Returns None when the
     operands do not qualify (dtype, alignment, no slack behind them): the caller then takes the
-    route over transposed copies."""
+    route over transposed copies.  ``halves``: dout holds the row gradients of two matrices side
+    by side; the result is two tensors [E, N/2, K_in] (fmoe_gemm_desc.out2)."""
     if dout.dtype != torch.bfloat16 or a_rows.dtype != torch.bfloat16 or dout.shape[0] != a_rows.shape[0]:
         return None
     R, N = dout.shape
@@ -209,15 +210,22 @@ def jagged_weight_grad(dout: torch.Tensor, a_rows: torch.Tensor, offsets: torch.
     ok = (dout.stride(1) == 1 and a_rows.stride(1) == 1 and N % 8 == 0 and Kin % 8 == 0 and E <= 256
           and dout.stride(0) % 8 == 0 and a_rows.stride(0) % 8 == 0 and dout.data_ptr() % 16 == 0
           and a_rows.data_ptr() % 16 == 0 and R >= 128 and E * N < (1 << 31)
-          and slack_rows(dout) >= SLACK_ROWS and slack_rows(a_rows) >= SLACK_ROWS)
+          and slack_rows(dout) >= SLACK_ROWS and slack_rows(a_rows) >= SLACK_ROWS
+          and (not halves or N % 64 == 0))
     if not ok:
         return None
     dev = dout.device
     offsets = _i64("offsets", offsets)
     seg = torch.arange(E + 1, device=dev, dtype=torch.int64) * N
-    out = torch.empty((E * N, Kin), dtype=torch.bfloat16, device=dev)
+    if halves:
+        out = torch.empty((E * (N // 2), Kin), dtype=torch.bfloat16, device=dev)
+        out2 = torch.empty_like(out)
+    else:
+        out = torch.empty((E * N, Kin), dtype=torch.bfloat16, device=dev)
     d = GemmDesc()
     d.num_experts, d.n, d.k, d.index_div = E, Kin, R, 1
+    if halves:
+        d.out2 = out2.data_ptr()
     d.total_rows, d.a_rows = E * N, N
     d.offsets = seg.data_ptr()
     d.a, d.a_dtype, d.a_stride_row, d.a_stride_k = dout.data_ptr(), _DTYPE_CODE[dout.dtype], 1, dout.stride(0)
@@ -227,6 +235,8 @@ def jagged_weight_grad(dout: torch.Tensor, a_rows: torch.Tensor, offsets: torch.
     d.k_window, d.k_slack_rows = offsets.data_ptr(), SLACK_ROWS
     rc = _lib.load().fmoe_grouped_gemm(ctypes.byref(d), _stream(dout))
     _lib.check(rc, "fmoe_grouped_gemm")
+    if halves:
+        return out.view(E, N // 2, Kin), out2.view(E, N // 2, Kin)
     return out.view(E, N, Kin)
 
 
@@ -494,21 +504,44 @@ def segment_colsum(src: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def swiglu_bwd(g: torch.Tensor, u: Optional[torch.Tensor], dh: torch.Tensor):
-    """Backward of ``silu(g) * u`` (or of ``silu(g)`` when u is None): returns (dg, du)."""
+def swiglu_bwd(g: torch.Tensor, u: Optional[torch.Tensor], dh: torch.Tensor, joint: bool = False):
+    """Backward of ``silu(g) * u`` (or of ``silu(g)`` when u is None): returns (dg, du).
+    ``joint`` (gated form, 2-D bf16, columns a multiple of 8): dg and du are the two halves of one
+    [rows, 2 * cols] buffer, ``torch.cat([dg, du], 1)`` without the copy, so that the GEMMs that
+    consume both can take them as one operand (``dg._base`` is that buffer's storage)."""
     _need_cuda("swiglu_bwd", g, u, dh)
     if g.dtype not in _DTYPE_CODE or dh.dtype != g.dtype or dh.shape != g.shape or (
             u is not None and (u.dtype != g.dtype or u.shape != g.shape)):
         raise ValueError("swiglu_bwd: bf16 (or fp32) tensors of one shape expected")
     g, dh = g.contiguous(), dh.contiguous()
     u = None if u is None else u.contiguous()
-    dg = empty_rows(g.shape[0], g.shape[1], g.dtype, g.device) if g.ndim == 2 else torch.empty_like(g)
-    du = None if u is None else (empty_rows(g.shape[0], g.shape[1], g.dtype, g.device) if g.ndim == 2
-                                 else torch.empty_like(g))
+    cols = g.shape[-1] if g.ndim >= 1 else 1
+    pitch = 0
+    if (joint and u is not None and g.ndim == 2 and g.dtype == torch.bfloat16 and cols % 8 == 0 and cols >= 8
+            and g.numel() > 0):
+        both = empty_rows(g.shape[0], 2 * cols, g.dtype, g.device)
+        dg, du, pitch = both[:, :cols], both[:, cols:], 2 * cols
+    else:
+        dg = empty_rows(g.shape[0], g.shape[1], g.dtype, g.device) if g.ndim == 2 else torch.empty_like(g)
+        du = None if u is None else (empty_rows(g.shape[0], g.shape[1], g.dtype, g.device) if g.ndim == 2
+                                     else torch.empty_like(g))
     rc = _lib.load().fmoe_swiglu_bwd(g.data_ptr(), _ptr(u), dh.data_ptr(), dg.data_ptr(), _ptr(du),
-                                     _DTYPE_CODE[g.dtype], g.numel(), _stream(g))
+                                     _DTYPE_CODE[g.dtype], g.numel(), cols, pitch, _stream(g))
     _lib.check(rc, "fmoe_swiglu_bwd")
     return dg, du
+
+
+def joint_rows(left: torch.Tensor, right: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """[rows, 2 * cols] view over two [rows, cols] tensors that are the halves of one buffer (what
+    ``swiglu_bwd(joint=True)`` returns), else None."""
+    if (right is None or left.ndim != 2 or left.shape != right.shape or left.dtype != right.dtype
+            or left.untyped_storage().data_ptr() != right.untyped_storage().data_ptr()):
+        return None
+    rows, cols = left.shape
+    if (left.stride() != (2 * cols, 1) or right.stride() != (2 * cols, 1)
+            or right.storage_offset() != left.storage_offset() + cols):
+        return None
+    return torch.as_strided(left, (rows, 2 * cols), (2 * cols, 1))
 
 
 def combine_bwd(dy: torch.Tensor, value: Optional[torch.Tensor], token_index: torch.Tensor, K: int,

@@ -230,6 +230,13 @@ typedef struct fmoe_gemm_desc {
                                 descriptors with a2 are turned away with FMOE_ERR_ARGUMENT */
     int32_t k2;             /* contraction length of a2 * b2                                */
     int32_t reserved1;
+    void* out2;             /* NULL, or (with a_stride_k only) a second output: offsets then
+                                describes experts of 2 * h rows each (h a multiple of 32), and
+                                rows [h, 2h) of every expert are stored to out2 + (e * h + row - h) *
+                                out_stride_row, rows [0, h) to out + (e * h + row) * out_stride_row:
+                                the weight gradients of two matrices (SwiGLU's gate and up
+                                projection, whose row gradients lie side by side) from one GEMM,
+                                each into its own [E, h, n] tensor                          */
 } fmoe_gemm_desc;
 
 int fmoe_grouped_gemm(const fmoe_gemm_desc* desc /* host pointer */, fmoe_stream_t stream);
@@ -327,9 +334,14 @@ int fmoe_segment_colsum(const void* src, int dtype, int64_t total_rows, int64_t 
  *   du = dh * silu(g),   dg = (dh * u) * sigmoid(g) * (1 + g * (1 - sigmoid(g)))
  * rounded where torch autograd rounds (silu(g), dh * u and both results in `dtype`).
  * u == NULL: plain SiLU backward, dg = dh * sigmoid(g) * (1 + g * (1 - sigmoid(g))), du unused.
+ * g, u, dh are contiguous with n elements.  out_stride_row = 0 (or = cols): so are dg and du.
+ * Otherwise the n elements are rows of `cols`, and row i of dg / du starts at element
+ * i * out_stride_row: the two halves of one [rows, 2 * cols] buffer (dg = buf, du = buf + cols,
+ * pitch 2 * cols), which the next GEMMs then read as one operand (bf16, cols and the pitch in
+ * multiples of 8).
  */
 int fmoe_swiglu_bwd(const void* g, const void* u, const void* dh, void* dg, void* du, int dtype,
-                    int64_t n, fmoe_stream_t stream);
+                    int64_t n, int64_t cols, int64_t out_stride_row, fmoe_stream_t stream);
 
 /*
  * Backward of fmoe_combine (kernels/triton/triton_moe.py:922-983): for every routed row r with

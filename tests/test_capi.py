@@ -107,6 +107,10 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
     assert b"a2 needs b2" in lib.fmoe_last_error()
     d.a2, d.k2 = None, 0
+    d.out2 = 64                              # a second output belongs to the row-indexed weight-gradient form
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
+    assert b"out2 goes with a_stride_k" in lib.fmoe_last_error()
+    d.out2 = None
     d.total_rows = 0
     assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 0 and plan.value == -1
     # routing: K > E, K > 64, workspace too small
@@ -128,7 +132,9 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert lib.fmoe_jagged_transpose(P, 1, 8, 8, 4, None, 1, P, P, 2, P, 16, 16, 0, None) == 1
     assert b"row stride" in lib.fmoe_last_error()
     assert lib.fmoe_segment_colsum(P, 1, 8, 8, 4, P, 2, P, None) == 1
-    assert lib.fmoe_swiglu_bwd(P, P, P, P, None, 1, 8, None) == 1          # gated form needs du
+    assert lib.fmoe_swiglu_bwd(P, P, P, P, None, 1, 8, 8, 0, None) == 1    # gated form needs du
+    assert lib.fmoe_swiglu_bwd(P, P, P, P, P, 0, 64, 8, 16, None) == 1     # pitched outputs: bf16 only
+    assert b"row pitch" in lib.fmoe_last_error()
     assert lib.fmoe_combine_bwd(P, None, 1, 4, 2, 8, 8, P, None, 0, 1, 1, 1, None, P,
                                 ctypes.cast(P, ctypes.POINTER(ctypes.c_float)), None) == 1
     assert b"d_gates needs value" in lib.fmoe_last_error()

@@ -581,3 +581,35 @@ def test_silu_backward_at_the_reference_sizes(N, dtype):
     dg, du = ops.swiglu_bwd(x.detach().view(-1, 1024), u.detach().view(-1, 1024), dy.view(-1, 1024))
     torch.testing.assert_close(dg.view(-1), x.grad)
     torch.testing.assert_close(du.view(-1), u.grad)
+
+
+@pytest.mark.parametrize("lens,H", [
+    ([900, 0, 513, 130, 64, 1, 300], 96),        # 2H = 192: one row tile per expert straddles both halves
+    ([2000, 129, 700], 352),                     # 2H = 704: the halves meet inside the second tile of three
+])
+def test_two_weight_gradients_from_one_gemm(lens, H):
+    """The row gradients of two matrices side by side in one buffer (what swiglu_bwd(joint=True)
+    writes): one GEMM stores each matrix's gradient into its own tensor (fmoe_gemm_desc.out2),
+    bit-identical to one GEMM per matrix on the halves."""
+    from fast_moe_amd.kernels.hip import ops
+    E, Kin = len(lens), 392
+    g = torch.Generator().manual_seed(5)
+    offsets = torch.zeros(E + 1, dtype=torch.int64)
+    offsets[1:] = torch.cumsum(torch.tensor(lens), 0)
+    R = int(offsets[-1])
+    xg, both = ops.empty_rows(R, Kin, BF16, "cuda"), ops.empty_rows(R, 2 * H, BF16, "cuda")
+    xg.copy_((torch.randn(R, Kin, generator=g) * 0.5).to(BF16))
+    both.copy_((torch.randn(R, 2 * H, generator=g) * 0.5).to(BF16))
+    left, right = both[:, :H], both[:, H:]
+    assert ops.joint_rows(left, right) is not None and ops.joint_rows(left, left) is None
+    pair = ops.jagged_weight_grad(both, xg, offsets.cuda(), halves=True)
+    assert pair is not None and all(t.is_contiguous() and tuple(t.shape) == (E, H, Kin) for t in pair)
+    one, two = ops.jagged_weight_grad(left, xg, offsets.cuda()), ops.jagged_weight_grad(right, xg, offsets.cuda())
+    assert one is not None and two is not None
+    assert torch.equal(pair[0], one) and torch.equal(pair[1], two)
+    # swiglu_bwd writes such a buffer: same values as the separate form
+    a, b, c = (torch.randn(R, H, generator=g).to(BF16).cuda() for _ in range(3))
+    dg, du = ops.swiglu_bwd(a, b, c, joint=True)
+    dg0, du0 = ops.swiglu_bwd(a, b, c)
+    assert ops.joint_rows(dg, du) is not None and ops.joint_rows(dg0, du0) is None
+    assert torch.equal(dg, dg0) and torch.equal(du, du0)
