@@ -239,6 +239,22 @@ __global__ __launch_bounds__(256) void swiglu_bwd_bf16x8_kernel(const uint16_t* 
     if (GATED) reinterpret_cast<u32x4*>(du)[o] = ou;
 }
 
+// dst[i, :] = src[index[i] / index_div, :] for rows of whole 16-byte chunks: one wavefront per
+// output row, ordinary (cached) loads, since a top-k router names every source row k times.
+__global__ __launch_bounds__(256) void gather_rows_kernel(const u32x4* __restrict__ src, int64_t src_rows,
+                                                          int64_t chunks, int64_t src_stride,
+                                                          const int64_t* __restrict__ index, int index_div,
+                                                          int64_t n_out, u32x4* __restrict__ dst,
+                                                          int64_t dst_stride) {
+    const int64_t row = (int64_t)blockIdx.x * 4 + threadIdx.x / kWave;
+    if (row >= n_out) return;
+    int64_t s = index[row] / index_div;
+    s = s < 0 ? 0 : (s >= src_rows ? src_rows - 1 : s);       // malformed index: clamped, never followed
+    const u32x4* from = src + s * src_stride;
+    u32x4* to = dst + row * dst_stride;
+    for (int64_t c = lane_id(); c < chunks; c += kWave) to[c] = from[c];
+}
+
 struct GateArgs {
     const void* ptr;
     int64_t cols, stride_row, stride_col;
@@ -342,6 +358,24 @@ extern "C" int fmoe_jagged_transpose(const void* src, int dtype, int64_t src_row
             (const float*)src, src_rows, cols, src_stride_row, row_index, index_div, offsets, pad_offsets,
             num_experts, (float*)dst, dst_stride, dst_cols, apply_silu);
     return check_launch("fmoe_jagged_transpose");
+}
+
+extern "C" int fmoe_gather_rows(const void* src, int64_t src_rows, int64_t row_bytes, int64_t src_stride_bytes,
+                                const int64_t* index, int index_div, int64_t n_out, void* dst,
+                                int64_t dst_stride_bytes, fmoe_stream_t stream) {
+    FMOE_REQUIRE(src_rows >= 0 && row_bytes >= 0 && n_out >= 0 && index_div >= 1,
+                 "fmoe_gather_rows: negative extent or index_div < 1");
+    if (n_out == 0 || row_bytes == 0) return FMOE_OK;
+    FMOE_REQUIRE(src && index && dst && src_rows >= 1, "fmoe_gather_rows: NULL pointer or no source rows");
+    FMOE_REQUIRE(row_bytes % 16 == 0 && src_stride_bytes % 16 == 0 && dst_stride_bytes % 16 == 0 && aligned16(src) &&
+                     aligned16(dst) && src_stride_bytes >= row_bytes && dst_stride_bytes >= row_bytes,
+                 "fmoe_gather_rows: rows and row pitches are whole, 16-byte aligned chunks (row_bytes=%lld)",
+                 (long long)row_bytes);
+    FMOE_REQUIRE((n_out + 3) / 4 < ((int64_t)1 << 31), "fmoe_gather_rows: too many rows");
+    gather_rows_kernel<<<(unsigned)((n_out + 3) / 4), 256, 0, (hipStream_t)stream>>>(
+        (const u32x4*)src, src_rows, row_bytes / 16, src_stride_bytes / 16, index, index_div, n_out, (u32x4*)dst,
+        dst_stride_bytes / 16);
+    return check_launch("fmoe_gather_rows");
 }
 
 extern "C" int fmoe_segment_colsum(const void* src, int dtype, int64_t total_rows, int64_t cols,

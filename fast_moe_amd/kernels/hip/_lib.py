@@ -22,7 +22,7 @@ EXPORTED_SYMBOLS = (
     "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_grouped_gemm_plan",
     "fmoe_combine",
     "fmoe_silu_mul", "fmoe_transpose_last2", "fmoe_jagged_transpose", "fmoe_segment_colsum",
-    "fmoe_swiglu_bwd", "fmoe_combine_bwd",
+    "fmoe_swiglu_bwd", "fmoe_combine_bwd", "fmoe_gather_rows",
 )
 
 
@@ -97,6 +97,9 @@ def load() -> ctypes.CDLL:
     lib.fmoe_segment_colsum.restype = c_int
     lib.fmoe_segment_colsum.argtypes = [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p,
                                         c_void_p]
+    lib.fmoe_gather_rows.restype = c_int
+    lib.fmoe_gather_rows.argtypes = [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p,
+                                     c_int64, c_void_p]
     lib.fmoe_swiglu_bwd.restype = c_int
     lib.fmoe_swiglu_bwd.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
                                     c_int64, c_void_p]

@@ -64,14 +64,14 @@ class _WgradOperand:
         self.args = (a_src, total_rows, row_index, index_div, apply_silu)
         self.rows = None            # [total_rows, K_in] in expert order, with slack
         self.a_t = None
-        if a_src.dtype == torch.bfloat16 and a_src.ndim == 2:
+        if a_src.dtype == torch.bfloat16 and a_src.ndim == 2 and a_src.shape[1] % 8 == 0:
             if row_index is None and not apply_silu:
                 self.rows = a_src
             elif row_index is None:             # SiLU with the rounding of F.silu on a bf16 tensor
                 self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
                 torch.ops.aten.silu.out(a_src, out=self.rows)
             elif not apply_silu:
-                self.rows = ops.gather_rows(a_src, torch.div(row_index, index_div, rounding_mode="floor"))
+                self.rows = ops.gather_rows(a_src, row_index, index_div)
 
     def _transposed(self):
         if self.a_t is None:

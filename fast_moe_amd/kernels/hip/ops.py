@@ -408,9 +408,8 @@ def gemm_plan(d: GemmDesc) -> int:
 
 # ------------------------------------------------------------------ combine
 def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[torch.Tensor] = None,
-            gates_index: Optional[torch.Tensor] = None, with_slack: bool = False) -> torch.Tensor:
-    """Weighted merge, see fmoe_combine.  value [T*K, D]; reverse_index [T, K].  ``with_slack``:
-    the output gets SLACK_ROWS readable rows behind it (see empty_rows)."""
+            gates_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Weighted merge, see fmoe_combine.  value [T*K, D]; reverse_index [T, K]."""
     dev = _need_cuda("combine", value, reverse_index, gates, gates_index)
     if value.dtype not in _DTYPE_CODE:
         raise NotImplementedError(f"combine: value must be fp32 or bf16, got {value.dtype}")
@@ -437,7 +436,7 @@ def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[to
                 raise ValueError("combine: gates_index must have T*K entries")
     else:
         gates_index = None
-    out = empty_rows(T, D, out_dtype, dev) if with_slack else torch.empty((T, D), dtype=out_dtype, device=dev)
+    out = torch.empty((T, D), dtype=out_dtype, device=dev)
     rc = _lib.load().fmoe_combine(
         value.data_ptr(), _DTYPE_CODE[value.dtype], T, K, D, value.stride(0), reverse_index.data_ptr(),
         _ptr(gates), g_code, g_cols, g_sr, g_sc, _ptr(gates_index), out.data_ptr(), _DTYPE_CODE[out_dtype],
@@ -446,10 +445,21 @@ def combine(value: torch.Tensor, reverse_index: torch.Tensor, gates: Optional[to
     return out
 
 
-def gather_rows(src: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
-    """``src[rows]`` for a 2-D src, as the K = 1 case of the merge kernel (one row per output row,
-    no weights); the result has slack rows behind it."""
-    return combine(src, rows.view(-1, 1), with_slack=True)
+def gather_rows(src: torch.Tensor, index: torch.Tensor, index_div: int = 1) -> torch.Tensor:
+    """``src[index // index_div]`` for a 2-D src with contiguous rows of whole 16-byte chunks
+    (fmoe_gather_rows); the result has slack rows behind it."""
+    dev = _need_cuda("gather_rows", src, index)
+    if src.ndim != 2:
+        raise ValueError("gather_rows: src must be 2-D")
+    src = _rows_contiguous(src)
+    index = _i64("index", index).view(-1)
+    out = empty_rows(index.numel(), src.shape[1], src.dtype, dev)
+    es = src.element_size()
+    rc = _lib.load().fmoe_gather_rows(src.data_ptr(), src.shape[0], src.shape[1] * es, src.stride(0) * es,
+                                      index.data_ptr(), index_div, index.numel(), out.data_ptr(),
+                                      out.stride(0) * es, _stream(src))
+    _lib.check(rc, "fmoe_gather_rows")
+    return out
 
 
 def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:

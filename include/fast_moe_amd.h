@@ -325,6 +325,16 @@ int fmoe_jagged_transpose(const void* src, int dtype, int64_t src_rows, int64_t 
  * fixed order: the bias gradient of the grouped GEMMs (torch autograd's sum over the rows of
  * each F.linear call in kernels/pytorch/moe.py:75-82).  src / out FMOE_BF16 or FMOE_F32.
  */
+/*
+ * dst[i, :] = src[index[i] / index_div, :]: the routed rows' inputs in expert order, what the
+ * weight-gradient GEMM contracts with (triton_index_select, kernels/triton/triton_general_ops.py:42-129,
+ * as called at kernels/triton/triton_moe.py:2451-2453).  Rows are row_bytes long (a multiple of
+ * 16, any element type), pitches in bytes; an index outside [0, src_rows) is clamped.
+ */
+int fmoe_gather_rows(const void* src, int64_t src_rows, int64_t row_bytes, int64_t src_stride_bytes,
+                     const int64_t* index, int index_div, int64_t n_out, void* dst,
+                     int64_t dst_stride_bytes, fmoe_stream_t stream);
+
 int fmoe_segment_colsum(const void* src, int dtype, int64_t total_rows, int64_t cols,
                         int64_t src_stride_row, const int64_t* offsets, int num_experts, void* out,
                         fmoe_stream_t stream);

@@ -131,6 +131,8 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert b"bf16 or fp32" in lib.fmoe_last_error()
     assert lib.fmoe_jagged_transpose(P, 1, 8, 8, 4, None, 1, P, P, 2, P, 16, 16, 0, None) == 1
     assert b"row stride" in lib.fmoe_last_error()
+    assert lib.fmoe_gather_rows(P, 4, 24, 24, P, 1, 4, P, 24, None) == 1      # rows of whole 16-byte chunks
+    assert b"16-byte aligned chunks" in lib.fmoe_last_error()
     assert lib.fmoe_segment_colsum(P, 1, 8, 8, 4, P, 2, P, None) == 1
     assert lib.fmoe_swiglu_bwd(P, P, P, P, None, 1, 8, 8, 0, None) == 1    # gated form needs du
     assert lib.fmoe_swiglu_bwd(P, P, P, P, P, 0, 64, 8, 16, None) == 1     # pitched outputs: bf16 only

@@ -613,3 +613,17 @@ def test_two_weight_gradients_from_one_gemm(lens, H):
     dg0, du0 = ops.swiglu_bwd(a, b, c)
     assert ops.joint_rows(dg, du) is not None and ops.joint_rows(dg0, du0) is None
     assert torch.equal(dg, dg0) and torch.equal(du, du0)
+
+
+@pytest.mark.parametrize("dtype,cols", [(BF16, 264), (torch.float32, 36), (torch.uint8, 48)])
+def test_gather_rows(dtype, cols):
+    """fmoe_gather_rows against torch indexing, bit for bit; indices outside the source are clamped."""
+    from fast_moe_amd.kernels.hip import ops
+    g = torch.Generator().manual_seed(2)
+    src = (torch.randn(300, cols, generator=g) * 50).to(dtype).cuda()
+    idx = torch.randint(0, 300 * 4, (5000,), generator=g).cuda()
+    out = ops.gather_rows(src, idx, 4)
+    assert torch.equal(out, src[idx // 4]) and ops.slack_rows(out) >= ops.SLACK_ROWS
+    bad = torch.tensor([-5, 10 ** 9, 7]).cuda()
+    assert torch.equal(ops.gather_rows(src, bad), src[torch.tensor([0, 299, 7]).cuda()])
+    assert ops.gather_rows(src, idx[:0]).shape == (0, cols)
