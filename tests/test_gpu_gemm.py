@@ -580,3 +580,52 @@ def test_reference_grouped_gemm_grid(G, M, K, fp8):
             ref = a[lo:hi].float() @ w[e].float()
             atol = 1e-5 + 4e-3 * K ** 0.5
         torch.testing.assert_close(out[lo:hi].float(), ref.to(BF16).float(), atol=atol, rtol=1.6e-2)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_seeded_random_shapes_all_operators(seed):
+    """A seeded draw of sizes in the spirit of the reference's hypothesis grids
+    (kernels/tests/moe_test.py:27-57, 401-423, 729-751): token counts, expert counts, top-k, widths
+    (multiples of 8 and not), weight layouts and bias, for the plain, SwiGLU and merge operators,
+    forward against the oracle and, on every third draw, backward as well."""
+    import random
+    from fast_moe_amd.kernels import moe
+    rnd = random.Random(1000 + seed)
+    E = rnd.choice([1, 2, 3, 8, 17, 40, 70])
+    K = rnd.randint(1, min(E, 4))
+    L = rnd.choice([1, 7, 64, 333, 1500, 5000])
+    Din = rnd.choice([8, 24, 40, 72, 128, 200, 256, 520]) + rnd.choice([0, 0, 0, 3])
+    Dout = rnd.choice([8, 16, 56, 128, 136, 256, 264]) + rnd.choice([0, 0, 0, 5])
+    contiguous, has_bias = rnd.random() < 0.5, rnd.random() < 0.5
+    r = make_routing(L, E, K, seed=seed)
+    x = randn((L, Din), seed + 1)
+    w = weights(E, Din, Dout, seed + 2, contiguous, scale=Din ** -0.5)
+    wp = weights(E, Din, Dout, seed + 3, contiguous, scale=Din ** -0.5)
+    b = randn((E, Dout), seed + 4) if has_bias else None
+    gates = torch.rand((L, K), generator=torch.Generator().manual_seed(seed)).to(BF16)
+    tag = f"seed {seed}: L={L} E={E} K={K} Din={Din} Dout={Dout} contiguous={contiguous} bias={has_bias}"
+    f32 = lambda t: None if t is None else t.float()
+    ref_plain = o_moe.index_select_jagged_bmm(r["offsets"], r["index"], f32(x), f32(w), f32(b))
+    ref_glu = o_moe.index_select_jagged_bmm_swiglu(r["offsets"], r["index"], f32(x), f32(w), f32(b), f32(wp), f32(b))
+    ref_merge = o_moe.mul_merge_k_add(r["token_index"], ref_plain.to(BF16), K, gates, r["gate_index"])
+    d = lambda t: None if t is None else dev(t)
+    with torch.no_grad():
+        plain = moe.index_select_jagged_bmm(0, d(r["offsets"]), d(r["index"]), d(x), d(w), d(b))
+        glu = moe.index_select_jagged_bmm_swiglu(0, d(r["offsets"]), d(r["index"]), d(x), d(w), d(b), d(wp), d(b))
+        merged = moe.mul_merge_k_add(d(r["token_index"]), d(r["reverse_index"]), d(ref_plain.to(BF16)),
+                                     weight=d(gates), weight_index=d(r["gate_index"]))
+    assert_bf16_close(plain, ref_plain, rtol=1.6e-2, atol=2e-2, what="plain " + tag)
+    assert_bf16_close(glu, ref_glu, rtol=1.6e-2, atol=2e-2, what="swiglu " + tag)
+    assert torch.equal(merged.cpu(), ref_merge), "merge " + tag
+    if seed % 3:
+        return
+    leaves_ref = [t.float().requires_grad_(True) for t in (x, w, wp)]
+    dout = randn((L * K, Dout), seed + 5) * 0.01
+    o_moe.index_select_jagged_bmm_swiglu(r["offsets"], r["index"], leaves_ref[0], leaves_ref[1], f32(b), leaves_ref[2],
+                                         f32(b)).backward(dout.float())
+    leaves = [dev(t).requires_grad_(True) for t in (x, w, wp)]
+    moe.index_select_jagged_bmm_swiglu(0, d(r["offsets"]), d(r["index"]), leaves[0], leaves[1], d(b), leaves[2],
+                                       d(b)).backward(dev(dout))
+    for name, got, ref in zip(("d_x", "d_w", "d_wp"), leaves, leaves_ref):
+        err = (got.grad.float().cpu() - ref.grad).abs().max().item()
+        assert err <= 3e-2 * ref.grad.abs().max().item() + 1e-6, (name, tag, err, ref.grad.abs().max().item())
