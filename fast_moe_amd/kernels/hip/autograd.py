@@ -5,15 +5,22 @@ What the reference's Triton autograd functions compute
 :62-141 fused SwiGLU backward, :922-983 merge backward, :3790-4027 silu_jagged_bmm_combine
 backward), built from the library's kernels:
 
-* input gradient  = grouped GEMM of the output gradient with the transposed weight, then the
+* input gradient  = grouped GEMM of the output gradient with the transposed weight (read in
+  place; the two branches of a SwiGLU layer summed in one GEMM, fmoe_gemm_desc.a2), then the
   deterministic gather-form sum of the K routed rows of every token (fmoe_combine);
-* weight gradient = grouped GEMM with a per-expert contraction window over the rows of the
-  expert (fmoe_grouped_gemm + k_window) on operands that fmoe_jagged_transpose laid out
-  K-contiguous and zero padded;
+* weight gradient = grouped GEMM over the rows of each expert as its contraction window
+  (fmoe_grouped_gemm + k_window), on the row-major tensors themselves (a_stride_k; the token
+  rows first put in expert order by fmoe_gather_rows; both matrices of a SwiGLU layer from one
+  launch, out2), or, for operands that do not qualify, on copies that fmoe_jagged_transpose
+  laid out K-contiguous and zero padded;
 * bias gradient   = fmoe_segment_colsum; activation and merge backward = fmoe_swiglu_bwd,
-  fmoe_combine_bwd.
+  fmoe_combine_bwd;
+* the e4m3 operators: backward in bf16 for silu_jagged_bmm_combine_fp8, on re-quantised e4m3
+  operands for index_select_jagged_bmm(fp8=True), as the reference's operators do.
 
-torch is used for index bookkeeping on [E]- and [T, K]-sized integer tensors only.
+Besides these kernels torch does index bookkeeping on [E]-, [R]- and [T, K]-sized integer
+tensors, the SiLU of saved rows where an operator was called with has_silu (aten.silu.out) and
+the fp32 index_add_ of the 3D variant's input gradient.
 """
 from __future__ import annotations
 
