@@ -23,14 +23,15 @@ int check_launch(const char* what) {
 
 namespace {
 
-// out = round(round(silu(a)) * b), 8 bf16 per thread
+// out = round(round(silu(a)) * b), 8 bf16 per thread; without b: out = round(silu(a))
+template <bool GATED>
 __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __restrict__ a,
                                                             const uint16_t* __restrict__ b,
                                                             uint16_t* __restrict__ out, int64_t n) {
     const int64_t i0 = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
-    if (i0 + 8 <= n && aligned_ok(a, b, out)) {
+    if (i0 + 8 <= n && aligned_ok(a, GATED ? b : a, out)) {
         const u32x4 va = *reinterpret_cast<const u32x4*>(a + i0);
-        const u32x4 vb = *reinterpret_cast<const u32x4*>(b + i0);
+        const u32x4 vb = GATED ? *reinterpret_cast<const u32x4*>(b + i0) : u32x4{0, 0, 0, 0};
         u32x4 vo;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __re
             for (int h = 0; h < 2; ++h) {
                 const float x = bf16_bits_to_f32((va[j] >> (16 * h)) & 0xffffu);
                 const float y = bf16_bits_to_f32((vb[j] >> (16 * h)) & 0xffffu);
-                r |= f32_to_bf16_bits(round_bf16(silu_f32(x)) * y) << (16 * h);
+                r |= f32_to_bf16_bits(GATED ? round_bf16(silu_f32(x)) * y : silu_f32(x)) << (16 * h);
             }
             vo[j] = r;
         }
@@ -47,17 +48,18 @@ __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __re
     } else {
         for (int64_t i = i0; i < n && i < i0 + 8; ++i) {
             const float x = bf16_bits_to_f32(a[i]);
-            const float y = bf16_bits_to_f32(b[i]);
-            out[i] = (uint16_t)f32_to_bf16_bits(round_bf16(silu_f32(x)) * y);
+            const float y = GATED ? bf16_bits_to_f32(b[i]) : 1.0f;
+            out[i] = (uint16_t)f32_to_bf16_bits(GATED ? round_bf16(silu_f32(x)) * y : silu_f32(x));
         }
     }
 }
 
+template <bool GATED>
 __global__ __launch_bounds__(256) void silu_mul_f32_kernel(const float* __restrict__ a,
                                                            const float* __restrict__ b,
                                                            float* __restrict__ out, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = silu_f32(a[i]) * b[i];
+    if (i < n) out[i] = GATED ? silu_f32(a[i]) * b[i] : silu_f32(a[i]);
 }
 
 // 64 x 64 tile transpose through LDS; reads and writes are both row-contiguous
@@ -116,14 +118,17 @@ extern "C" int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype,
     FMOE_REQUIRE(dtype == FMOE_BF16 || dtype == FMOE_F32, "fmoe_silu_mul: dtype must be bf16 or fp32");
     FMOE_REQUIRE(n >= 0, "fmoe_silu_mul: n < 0");
     if (n == 0) return FMOE_OK;
-    FMOE_REQUIRE(a && b && out, "fmoe_silu_mul: NULL pointer");
+    FMOE_REQUIRE(a && out, "fmoe_silu_mul: NULL pointer");
+    FMOE_REQUIRE((n + 255) / 256 < ((int64_t)1 << 31), "fmoe_silu_mul: too many elements");
+    hipStream_t s = (hipStream_t)stream;
     if (dtype == FMOE_F32) {
-        silu_mul_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(
-            (const float*)a, (const float*)b, (float*)out, n);
+        const unsigned blocks = (unsigned)((n + 255) / 256);
+        if (b) silu_mul_f32_kernel<true><<<blocks, 256, 0, s>>>((const float*)a, (const float*)b, (float*)out, n);
+        else silu_mul_f32_kernel<false><<<blocks, 256, 0, s>>>((const float*)a, nullptr, (float*)out, n);
         return check_launch("fmoe_silu_mul");
     }
-    const int64_t threads = (n + 7) / 8;
-    silu_mul_bf16_kernel<<<(unsigned)((threads + 255) / 256), 256, 0, (hipStream_t)stream>>>(
-        (const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, n);
+    const unsigned blocks = (unsigned)(((n + 7) / 8 + 255) / 256);
+    if (b) silu_mul_bf16_kernel<true><<<blocks, 256, 0, s>>>((const uint16_t*)a, (const uint16_t*)b, (uint16_t*)out, n);
+    else silu_mul_bf16_kernel<false><<<blocks, 256, 0, s>>>((const uint16_t*)a, nullptr, (uint16_t*)out, n);
     return check_launch("fmoe_silu_mul");
 }

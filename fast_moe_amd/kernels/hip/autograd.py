@@ -19,8 +19,7 @@ backward), built from the library's kernels:
   operands for index_select_jagged_bmm(fp8=True), as the reference's operators do.
 
 Besides these kernels torch does index bookkeeping on [E]-, [R]- and [T, K]-sized integer
-tensors, the SiLU of saved rows where an operator was called with has_silu (aten.silu.out) and
-the fp32 index_add_ of the 3D variant's input gradient.
+tensors and the fp32 index_add_ of the 3D variant's input gradient.
 """
 from __future__ import annotations
 
@@ -74,9 +73,8 @@ class _WgradOperand:
         if a_src.dtype == torch.bfloat16 and a_src.ndim == 2 and a_src.shape[1] % 8 == 0:
             if row_index is None and not apply_silu:
                 self.rows = a_src
-            elif row_index is None:             # SiLU with the rounding of F.silu on a bf16 tensor
-                self.rows = ops.empty_rows(total_rows, a_src.shape[1], a_src.dtype, a_src.device)
-                torch.ops.aten.silu.out(a_src, out=self.rows)
+            elif row_index is None:             # SiLU rounded as the forward GEMM rounds it on load
+                self.rows = ops.silu_mul(a_src, None, with_slack=True)
             elif not apply_silu:
                 self.rows = ops.gather_rows(a_src, row_index, index_div)
 

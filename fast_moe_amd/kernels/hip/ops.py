@@ -462,14 +462,16 @@ def gather_rows(src: torch.Tensor, index: torch.Tensor, index_div: int = 1) -> t
     return out
 
 
-def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """``silu(a) * b`` element-wise (bf16 or fp32, same shape)."""
+def silu_mul(a: torch.Tensor, b: Optional[torch.Tensor], with_slack: bool = False) -> torch.Tensor:
+    """``silu(a) * b`` element-wise (bf16 or fp32, same shape); ``silu(a)`` when b is None.
+    ``with_slack`` (2-D a): the result has SLACK_ROWS readable rows behind it."""
     _need_cuda("silu_mul", a, b)
-    if a.dtype not in _DTYPE_CODE or b.dtype != a.dtype or a.shape != b.shape:
+    if a.dtype not in _DTYPE_CODE or (b is not None and (b.dtype != a.dtype or a.shape != b.shape)):
         raise ValueError("silu_mul: two bf16 (or two fp32) tensors of one shape expected")
-    a, b = a.contiguous(), b.contiguous()
-    out = torch.empty_like(a)
-    rc = _lib.load().fmoe_silu_mul(a.data_ptr(), b.data_ptr(), out.data_ptr(), _DTYPE_CODE[a.dtype], a.numel(),
+    a = a.contiguous()
+    b = None if b is None else b.contiguous()
+    out = empty_rows(a.shape[0], a.shape[1], a.dtype, a.device) if with_slack and a.ndim == 2 else torch.empty_like(a)
+    rc = _lib.load().fmoe_silu_mul(a.data_ptr(), _ptr(b), out.data_ptr(), _DTYPE_CODE[a.dtype], a.numel(),
                                    _stream(a))
     _lib.check(rc, "fmoe_silu_mul")
     return out

@@ -282,7 +282,9 @@ int fmoe_combine(const void* value, int value_dtype, int64_t T, int K, int64_t D
 
 /* out[i] = silu(a[i]) * b[i] over n bf16 (or fp32) elements with the reference's rounding
  * points (F.silu(alpha) * beta, kernels/pytorch/moe.py:221): the element-wise
- * tail of index_select_jagged_gating_bmm when its two inputs differ. */
+ * tail of index_select_jagged_gating_bmm when its two inputs differ.  b == NULL: out = silu(a)
+ * (F.silu in the operand's dtype, kernels/pytorch/moe.py:266), the rows the weight gradient of
+ * silu_jagged_bmm_combine(has_silu=True) contracts with. */
 int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
                   fmoe_stream_t stream);
 

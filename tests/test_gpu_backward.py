@@ -627,3 +627,18 @@ def test_gather_rows(dtype, cols):
     bad = torch.tensor([-5, 10 ** 9, 7]).cuda()
     assert torch.equal(ops.gather_rows(src, bad), src[torch.tensor([0, 299, 7]).cuda()])
     assert ops.gather_rows(src, idx[:0]).shape == (0, cols)
+
+
+@pytest.mark.parametrize("dtype", [BF16, torch.float32])
+def test_silu_mul_and_its_plain_form(dtype):
+    """fmoe_silu_mul against torch on the GPU: the gated form with the rounding points of
+    F.silu(a) * b, the plain form (b = NULL) against F.silu; odd lengths take the scalar tail."""
+    from fast_moe_amd.kernels.hip import ops
+    g = torch.Generator(device="cuda").manual_seed(1)
+    for shape in ((257, 1031), (64, 1408)):
+        a = torch.randn(shape, device="cuda", generator=g).to(dtype) * 3
+        b = torch.randn(shape, device="cuda", generator=g).to(dtype)
+        torch.testing.assert_close(ops.silu_mul(a, b), torch.nn.functional.silu(a) * b)
+        plain = ops.silu_mul(a, None, with_slack=True)
+        torch.testing.assert_close(plain, torch.nn.functional.silu(a))
+        assert ops.slack_rows(plain) >= ops.SLACK_ROWS
