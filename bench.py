@@ -311,6 +311,47 @@ def run_train(w, steps, warmup):
     return ms, ms_fwd, 3.0 * (f1 + f2)
 
 
+def run_sgmoe(steps, warmup, tokens):
+    """The SGMoE layer with the MRN router front-end at the 64-expert top-8 size of
+    the headline workload (SiLU MLP experts, as the layer has them): evaluation forward,
+    training step, and the share of the router front-end (norm, normalised-logit gating,
+    dispatch) in the forward.  Reported beside the forward metric, never instead of it."""
+    from fast_moe_amd.modules.sgmoe import SGConfig, SGMoE
+    dev = torch.device("cuda:0")
+    T, D, H, E, K = tokens, 2048, 1408, 64, 8
+    torch.manual_seed(0)
+    layer = SGMoE(D, D, False, 1, SGConfig(model_d=H, num_experts=E, num_activated_experts=K)).to(dev).to(torch.bfloat16)
+    x = torch.randn(T, D, device=dev).to(torch.bfloat16)
+    dy = torch.randn(T, D, device=dev).to(torch.bfloat16) * 0.01
+    stream = torch.cuda.current_stream(dev)
+
+    def front_end():
+        x_norm = torch.nn.functional.layer_norm(x, (D,), layer._norm_w, layer._norm_bias, layer.norm_eps).to(x.dtype)
+        _, gates, idx, _ = layer._noisy_gating(x_norm, False, None)
+        from fast_moe_amd.kernels.hip import ops
+        return ops.route_from_topk(idx, E), gates
+
+    def train_step():
+        layer.zero_grad(set_to_none=True)
+        out = layer(x)
+        (out.x * dy).sum().add(out.loss.sum() if out.loss is not None else 0).backward()
+
+    layer.eval()
+    with torch.no_grad():
+        for _ in range(max(warmup, 1)):
+            layer(x)
+        torch.cuda.synchronize()
+        ms_eval = time_region(lambda: layer(x), steps, stream)
+        ms_front = time_region(front_end, steps, stream)
+    layer.train()
+    for _ in range(max(warmup, 1)):
+        train_step()
+    torch.cuda.synchronize()
+    ms_train = time_region(train_step, steps, stream)
+    flops = 2.0 * T * K * (D * H + H * D) + 2.0 * T * D * D       # routed experts + shared-expert addmm
+    return ms_eval, ms_front, ms_train, flops, (T, D, H, E, K)
+
+
 def bench_workload(name, steps, warmup, tokens=None):
     w = dict(WORKLOADS[name])
     if tokens:
@@ -330,6 +371,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary fp8 / bf16 workload")
     ap.add_argument("--backward", action="store_true",
                     help="time forward + backward of the bf16 SwiGLU workload instead of the forward metric")
+    ap.add_argument("--sgmoe", action="store_true",
+                    help="time the SGMoE layer (MRN router front-end + experts), forward and training step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 512 MiB device copy, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -341,6 +384,16 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
 
+    if args.sgmoe:
+        ms_eval, ms_front, ms_train, flops, (T, D, H, E, K) = run_sgmoe(args.steps, args.warmup, args.tokens or 16384)
+        print(json.dumps({
+            "metric": "sgmoe_forward_tflops", "value": round(flops / ms_eval / 1e9, 2), "unit": "TFLOP/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_eval, 4),
+            "ms_router_front_end": round(ms_front, 4), "ms_training_step": round(ms_train, 4),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": f"SGMoE layer (layer norm, normalised-logit router, SiLU MLP experts, shared-expert "
+                                   f"addmm), T={T}, E={E}, top-{K}, D={D}, H={H}"}}))
+        return
     if args.backward:
         w = dict(WORKLOADS[args.workload])
         if w["kind"] != "swiglu" or w["dtype"] != "bf16":

@@ -359,6 +359,16 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
         if b2 is not None:
             b2 = to_k_contiguous(b2)
             d.b2 = b2.data_ptr()
+    # SiLU on load exists in the register-staged kernel only.  Where the LDS-ring kernel would take
+    # the same call without it, one element-wise pass over the source rows (same rounding: SiLU in
+    # fp32, rounded to bf16 before it multiplies) and the ring kernel are faster together.
+    if a_silu and a.dtype == torch.bfloat16 and a.ndim == 2 and total_rows * N >= (1 << 22):
+        d.a_silu = 0
+        if gemm_plan(d) == _lib.PLAN_RING:
+            a = silu_mul(a, None)
+            d.a, d.a_stride_row = a.data_ptr(), a.stride(0)
+        else:
+            d.a_silu = 1
     rc = lib.fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
     _lib.check(rc, "fmoe_grouped_gemm")
     return out

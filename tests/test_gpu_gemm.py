@@ -629,3 +629,33 @@ def test_seeded_random_shapes_all_operators(seed):
     for name, got, ref in zip(("d_x", "d_w", "d_wp"), leaves, leaves_ref):
         err = (got.grad.float().cpu() - ref.grad).abs().max().item()
         assert err <= 3e-2 * ref.grad.abs().max().item() + 1e-6, (name, tag, err, ref.grad.abs().max().item())
+
+
+def test_silu_on_load_at_ring_size_takes_the_silu_pass():
+    """silu_jagged_bmm_combine(has_silu=True) large enough for the LDS-ring kernel: SiLU is applied by
+    an element-wise pass (the ring kernel has no SiLU on load) with the rounding of the staged
+    kernel's SiLU on load, so the GEMM input is bit-identical and the result meets the same bar."""
+    from fast_moe_amd.kernels import moe
+    from fast_moe_amd.kernels.hip import ops
+    T, E, K, H, O = 4096, 8, 2, 256, 512
+    r = make_routing(T, E, K, seed=21)
+    j = randn((T * K, H), 1)
+    w = weights(E, H, O, 2, False, scale=H ** -0.5)
+    b = randn((E, O), 3)
+    gates = torch.rand((T, K), generator=torch.Generator().manual_seed(4)).to(BF16)
+    ref = o_moe.silu_jagged_bmm_combine(r["offsets"], j.float(), w.float(), b.float(), r["token_index"], K,
+                                        gates.float(), r["gate_index"], True)
+    with torch.no_grad():
+        out = moe.silu_jagged_bmm_combine(0, dev(r["offsets"]), dev(j), dev(w), dev(b), dev(r["token_index"]),
+                                          dev(r["reverse_index"]), dev(gates), dev(r["gate_index"]), has_silu=True)
+        # the pass is what the caller could have done by hand
+        rows = ops.grouped_gemm(dev(r["offsets"]), dev(j), dev(w), total_rows=T * K, bias=dev(b), a_silu=True)
+        rows2 = ops.grouped_gemm(dev(r["offsets"]), ops.silu_mul(dev(j), None), dev(w), total_rows=T * K, bias=dev(b))
+        # ... and a slice small enough for the staged kernel's SiLU on load sees the same input bits
+        n_small = int(r["offsets"][1])
+        small = ops.grouped_gemm(dev(r["offsets"][:2]), dev(j[:n_small]), dev(w[:1]), total_rows=n_small,
+                                 bias=dev(b[:1]), a_silu=True)
+    assert torch.equal(rows, rows2)
+    assert_bf16_close(small, rows[:n_small].float(), rtol=1e-2, atol=1e-2, what="staged SiLU on load vs pass + ring")
+    scale = ref.abs().max().item()
+    assert_bf16_close(out, ref, rtol=1.6e-2, atol=1e-2 * scale, what="silu combine at ring size")
