@@ -16,6 +16,7 @@ import torch.nn.functional as F
 
 from ..kernels import moe
 from ..kernels.hip import ops
+from ..kernels.hip._lib import EPI_SILU
 from ..kernels.utils import KernelType
 from ..utils.utils import (_compute_top_logits, _create_fused_mlp_weights, _dispatch, _noisy_logits,
                            _prob_in_top_k, _train_loss, fx_torch_zeros)
@@ -101,6 +102,15 @@ class SGMoE(torch.nn.Module):
 
     def _expert_forward(self, x, token_index, offsets, reverse_index, gate_index, gating_scores):
         """mrn_test.py:292-327 without the host-side max_seq_len."""
+        if not torch.is_grad_enabled():
+            # inference: SiLU in the epilogue of the first GEMM (rounded to bf16 before and after the
+            # activation, as the two-operator form rounds it), no pass of its own
+            hidden = ops.grouped_gemm(offsets, x, self._experts_hidden_w.permute(0, 2, 1).to(x.dtype),
+                                      total_rows=gate_index.numel(), row_index=gate_index, index_div=self.k,
+                                      bias=self._experts_hidden_bias.to(x.dtype), epilogue=EPI_SILU)
+            return moe.silu_jagged_bmm_combine(
+                0, offsets, hidden, self._experts_w.permute(0, 2, 1).to(x.dtype), self._experts_bias.to(x.dtype),
+                token_index, reverse_index, gating_scores, gate_index, has_silu=False, kernel=KernelType.HIP)
         hidden = moe.index_select_jagged_bmm(
             0, offsets, gate_index.view(-1, self.k), x, self._experts_hidden_w.permute(0, 2, 1).to(x.dtype),
             self._experts_hidden_bias.to(x.dtype), kernel=KernelType.HIP)
