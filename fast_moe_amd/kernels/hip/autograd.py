@@ -361,23 +361,31 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
     @staticmethod
     def forward(ctx, offsets, jagged, weight, bias, index, reverse_index, gating_scores, gates_index, has_silu,
                 fp8_weight=None, recompute=False):
+        silu_rows = None
         if fp8_weight is None:
-            bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
-                                       epilogue=EPI_NONE, a_silu=has_silu)
+            if has_silu and not recompute and jagged.dtype == torch.bfloat16 and jagged.ndim == 2:
+                # SiLU once, kept for the weight gradient (the reference saves silu_jagged as well,
+                # kernels/triton/triton_moe.py:3770-3776); with recompute it is made again in backward
+                silu_rows = ops.silu_mul(jagged, None, with_slack=True)
+                bmm_out = ops.grouped_gemm(offsets, silu_rows, weight, total_rows=jagged.shape[0], bias=bias,
+                                           epilogue=EPI_NONE)
+            else:
+                bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
+                                           epilogue=EPI_NONE, a_silu=has_silu)
         else:
             qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
             bmm_out = ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=jagged.shape[0], bias=bias,
                                        a_scale=sa, b_scale=fp8_weight[1], epilogue=EPI_NONE)
         out = ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
         ctx.save_for_backward(offsets, jagged, weight, bias, index, gating_scores, gates_index,
-                              None if recompute else bmm_out)
+                              None if recompute else bmm_out, silu_rows)
         ctx.has_silu = has_silu
         ctx.K = reverse_index.shape[1]
         return out
 
     @staticmethod
     def backward(ctx, dy):
-        offsets, jagged, weight, bias, index, gating_scores, gates_index, bmm_out = ctx.saved_tensors
+        offsets, jagged, weight, bias, index, gating_scores, gates_index, bmm_out, silu_rows = ctx.saved_tensors
         if bmm_out is None:
             bmm_out = ops.grouped_gemm(offsets, jagged, weight, total_rows=jagged.shape[0], bias=bias,
                                        epilogue=EPI_NONE, a_silu=ctx.has_silu)
@@ -391,7 +399,10 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
             d_h = ops.grouped_gemm(offsets, d_bmm, weight.permute(0, 2, 1), total_rows=d_bmm.shape[0])
             d_jagged = ops.swiglu_bwd(jagged, None, d_h)[0] if ctx.has_silu else d_h
         if need[2]:
-            operand = _WgradOperand(jagged, offsets, jagged.shape[0], apply_silu=ctx.has_silu)
+            if silu_rows is not None:
+                operand = _WgradOperand(silu_rows, offsets, jagged.shape[0])
+            else:
+                operand = _WgradOperand(jagged, offsets, jagged.shape[0], apply_silu=ctx.has_silu)
             d_w = operand.weight_grad(d_bmm).permute(0, 2, 1)
         if bias is not None and need[3]:
             d_b = ops.segment_colsum(d_bmm, offsets)
