@@ -175,6 +175,69 @@ __global__ __launch_bounds__(256) void segment_colsum_kernel(const T* __restrict
     }
 }
 
+// bf16 rows of whole 16-byte chunks: one block per (expert, 64 columns) as above, but a lane
+// reads 8 columns at a time, 8 lanes cover the 128 bytes of a row segment and the 32 row lanes
+// of the block (8 per wave) take every 32nd row, four rows in flight per lane.  Sums in fp32 in
+// a fixed order: a lane's rows in ascending order, then the row lanes of a wave by a butterfly,
+// then the four waves.
+__global__ __launch_bounds__(256) void segment_colsum_bf16x8_kernel(const uint16_t* __restrict__ src,
+                                                                    int64_t total_rows, int64_t cols, int64_t stride,
+                                                                    const int64_t* __restrict__ offsets,
+                                                                    uint16_t* __restrict__ out) {
+    __shared__ float part[4][64];
+    const int e = blockIdx.y;
+    const int lane = lane_id(), wave = threadIdx.x / kWave;
+    const int cl = lane & 7, rl = wave * 8 + (lane >> 3);
+    const int64_t c = (int64_t)blockIdx.x * 64 + cl * 8;
+    int64_t lo = offsets[e], hi = offsets[e + 1];
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > total_rows ? total_rows : hi;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (c < cols) {
+        const uint16_t* col = src + c;
+        int64_t r = lo + rl;
+        for (; r + 96 < hi; r += 128) {
+            u32x4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = *reinterpret_cast<const u32x4*>(col + (r + 32 * i) * stride);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    acc[2 * j] += bf16_bits_to_f32(v[i][j] & 0xffffu);
+                    acc[2 * j + 1] += __uint_as_float(v[i][j] & 0xffff0000u);
+                }
+        }
+        for (; r < hi; r += 32) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(col + r * stride);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[2 * j] += bf16_bits_to_f32(v[j] & 0xffffu);
+                acc[2 * j + 1] += __uint_as_float(v[j] & 0xffff0000u);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float a = acc[j];
+        a += __shfl_xor(a, 8);
+        a += __shfl_xor(a, 16);
+        a += __shfl_xor(a, 32);
+        acc[j] = a;
+    }
+    if (lane < 8) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part[wave][lane * 8 + j] = acc[j];
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int64_t cc = (int64_t)blockIdx.x * 64 + threadIdx.x;
+        const int x = threadIdx.x;
+        if (cc < cols)
+            out[(int64_t)e * cols + cc] = (uint16_t)f32_to_bf16_bits((part[0][x] + part[1][x]) + (part[2][x] + part[3][x]));
+    }
+}
+
 __device__ __forceinline__ float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 template <typename T, bool GATED>
@@ -388,7 +451,10 @@ extern "C" int fmoe_segment_colsum(const void* src, int dtype, int64_t total_row
     FMOE_REQUIRE((src || total_rows == 0) && offsets && out, "fmoe_segment_colsum: NULL pointer");
     FMOE_REQUIRE(src_stride_row >= cols, "fmoe_segment_colsum: row stride shorter than the row");
     dim3 grid((unsigned)((cols + 63) / 64), (unsigned)num_experts);
-    if (dtype == FMOE_BF16)
+    if (dtype == FMOE_BF16 && cols % 8 == 0 && src_stride_row % 8 == 0 && aligned16(src))
+        segment_colsum_bf16x8_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(
+            (const uint16_t*)src, total_rows, cols, src_stride_row, offsets, (uint16_t*)out);
+    else if (dtype == FMOE_BF16)
         segment_colsum_kernel<uint16_t><<<grid, 256, 0, (hipStream_t)stream>>>(
             (const uint16_t*)src, total_rows, cols, src_stride_row, offsets, (uint16_t*)out);
     else

@@ -642,3 +642,29 @@ def test_silu_mul_and_its_plain_form(dtype):
         plain = ops.silu_mul(a, None, with_slack=True)
         torch.testing.assert_close(plain, torch.nn.functional.silu(a))
         assert ops.slack_rows(plain) >= ops.SLACK_ROWS
+
+
+@pytest.mark.parametrize("lens,cols,dtype", [
+    ([900, 0, 513, 4000, 1, 31, 32, 33, 127], 264, BF16),     # vector kernel, last column block 8 wide
+    ([20000, 3, 0, 777], 2048, BF16),                         # one long expert
+    ([300, 200, 0, 5], 20, BF16),                             # rows that are not whole 16-byte chunks
+    ([300, 200, 0, 5], 72, torch.float32),
+])
+def test_segment_colsum(lens, cols, dtype):
+    """fmoe_segment_colsum against per-expert fp32 sums (bias gradients); a pitched view as well."""
+    from fast_moe_amd.kernels.hip import ops
+    E, R = len(lens), sum(lens)
+    offsets = torch.tensor([0] + lens).cumsum(0)
+    src = (torch.randn(R, cols, generator=torch.Generator().manual_seed(7)) * 0.1).to(dtype)
+    ref = torch.stack([src[offsets[e]:offsets[e + 1]].double().sum(0) for e in range(E)])
+    out = ops.segment_colsum(src.cuda(), offsets.cuda())
+    assert out.dtype == dtype and tuple(out.shape) == (E, cols)
+    tol = 8e-3 if dtype == BF16 else 1e-5
+    err = (out.double().cpu() - ref).abs().max().item()
+    assert err <= tol * max(1.0, ref.abs().max().item()), err
+    assert not out[torch.tensor(lens) == 0].any()
+    if cols % 16 == 0:
+        wide = torch.zeros(R, 2 * cols, dtype=dtype)
+        wide[:, cols:] = src
+        again = ops.segment_colsum(wide.cuda()[:, cols:], offsets.cuda())
+        assert torch.equal(again, out)
