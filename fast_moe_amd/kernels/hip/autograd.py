@@ -18,8 +18,8 @@ backward), built from the library's kernels:
 * the e4m3 operators: backward in bf16 for silu_jagged_bmm_combine_fp8, on re-quantised e4m3
   operands for index_select_jagged_bmm(fp8=True), as the reference's operators do.
 
-Besides these kernels torch does index bookkeeping on [E]-, [R]- and [T, K]-sized integer
-tensors and the fp32 index_add_ of the 3D variant's input gradient.
+Besides these kernels torch does index bookkeeping only, on [E]-, [R]-, [T, K]- and (3D variant)
+[T, E, K]-sized integer tensors.
 """
 from __future__ import annotations
 
@@ -315,12 +315,16 @@ class IndexSelectJaggedBmm3D(torch.autograd.Function):
             cell = torch.div(index.reshape(-1), K, rounding_mode="floor") * E + expert
         if need[2]:
             d_rows = ops.grouped_gemm(offsets, dout, weight.permute(0, 2, 1), total_rows=R)
-            # every (token, expert) cell receives the rows routed there, most cells none: summed in
-            # fp32 as the reference does (:1412-1416, 1470); with the distinct experts per token
-            # of a top-k router each cell gets one row at most and the sum has one order
-            acc = torch.zeros((L * E, Kin), dtype=torch.float32, device=dout.device)
-            acc.index_add_(0, cell, d_rows.float())
-            d_jagged = acc.to(jagged.dtype).view(L, E, Kin)
+            # every (token, expert) cell receives the rows routed there, most cells none (the
+            # reference adds into an fp32 [L, A, E, K] tensor of zeros and sums it, :1412-1416, 1470).
+            # Gather form instead: slot j of cell (l, e) names the j-th routed row of token l if
+            # that row went to expert e, else nothing; the merge kernel adds a cell's rows in
+            # ascending order in fp32 and writes zeros where there are none.
+            rows_of_token = _reverse_from_index(index)                                  # [L, K] ascending
+            experts_of = expert[rows_of_token]                                          # [L, K]
+            here = experts_of[:, None, :] == torch.arange(E, device=index.device)[None, :, None]
+            slots = torch.where(here, rows_of_token[:, None, :], rows_of_token.new_full((), -1))
+            d_jagged = ops.combine(d_rows, slots.view(L * E, K)).view(L, E, Kin).to(jagged.dtype)
         if need[3]:
             src = jagged.contiguous().view(L * E, Kin)
             d_w = _WgradOperand(src, offsets, R, row_index=cell, index_div=1).weight_grad(dout).permute(0, 2, 1)

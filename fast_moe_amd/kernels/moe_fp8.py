@@ -131,8 +131,8 @@ def silu_jagged_bmm_fp8(
     require_hip_kernel(kernel, "silu_jagged_bmm_fp8")
     ops._forward_only("silu_jagged_bmm_fp8", jagged, weight, bias)
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=True)
-    qw, sw = ops.quant_rows_fp8(weight)                      # rows of [E, D_out, D_in]
-    return ops.grouped_gemm(seq_offsets, qa, qw.permute(0, 2, 1), total_rows=jagged.shape[0], bias=bias,
+    qw, sw = cached_quantize_expert_weights(weight.permute(0, 2, 1))    # rows of [E, D_out, D_in], once per update
+    return ops.grouped_gemm(seq_offsets, qa, qw, total_rows=jagged.shape[0], bias=bias,
                             a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
 
 

@@ -659,3 +659,33 @@ def test_silu_on_load_at_ring_size_takes_the_silu_pass():
     assert_bf16_close(small, rows[:n_small].float(), rtol=1e-2, atol=1e-2, what="staged SiLU on load vs pass + ring")
     scale = ref.abs().max().item()
     assert_bf16_close(out, ref, rtol=1.6e-2, atol=1e-2 * scale, what="silu combine at ring size")
+
+
+@pytest.mark.parametrize("lens,Din,Dout", [([300, 0, 77, 1000], 64, 32), ([2048, 4096], 256, 512)])
+def test_silu_jagged_bmm_fp8(lens, Din, Dout):
+    """moe_fp8.silu_jagged_bmm_fp8 (weight [E, D_out, D_in]): SiLU + row quantisation of the rows,
+    row quantisation of the weight, fp8 GEMM + bias, against the same composition of the oracle's
+    pieces (kernels/pytorch/moe_fp8.py:17-33, 127-137) and, loosely, the unquantised result the
+    reference's PyTorch path returns (:46-75); the second call hits the weight cache."""
+    from fast_moe_amd.kernels import moe_fp8
+    from oracle import fp8 as o_q
+    E, R = len(lens), sum(lens)
+    offsets = torch.tensor([0] + lens).cumsum(0)
+    j = randn((R, Din), 1)
+    w = randn((E, Dout, Din), 2, scale=Din ** -0.5)
+    b = randn((E, Dout), 3)
+    qa, sa = o_q.silu_rowwise_quant_fp8(j.float().numpy(), "bf16")
+    qw, sw = o_q.rowwise_quant_fp8(w.float().numpy(), "bf16")
+    qa_f, qw_f = torch.from_numpy(o_q.e4m3fn_decode(qa)), torch.from_numpy(o_q.e4m3fn_decode(qw))
+    rows = [qa_f[offsets[e]:offsets[e + 1]] for e in range(E)]
+    srow = [torch.from_numpy(sa)[offsets[e]:offsets[e + 1]] for e in range(E)]
+    ref = torch.cat(o_fp8.fp8_linear_per_expert(rows, srow, qw_f, torch.from_numpy(sw), b, BF16), dim=0)
+    with torch.no_grad():
+        out = moe_fp8.silu_jagged_bmm_fp8(dev(offsets), 0, dev(j), dev(w), dev(b))
+        again = moe_fp8.silu_jagged_bmm_fp8(dev(offsets), 0, dev(j), dev(w), dev(b))
+    assert torch.equal(out, again)
+    scale = ref.float().abs().max().item()
+    assert_bf16_close(out, ref.float(), rtol=1e-2, atol=1e-2 * scale, what="silu_jagged_bmm_fp8")
+    raw = torch.cat([torch.nn.functional.silu(j[offsets[e]:offsets[e + 1]].float()) @ w[e].float().T + b[e].float()
+                     for e in range(E)])
+    assert (out.float().cpu() - raw).abs().max().item() <= 0.1 * scale
