@@ -337,7 +337,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     uint16_t* obase = p.out + block_row * p.out_stride;
                     if constexpr (OUT2) {
                         if (p.out2) {       // (scalar arithmetic: everything here is wave-uniform)
-                            const int64_t m = block_row - (int64_t)expert * (2 * p.out_half);
+                            // (offsets that are not the promised e * 2h are not followed out of
+                            // the two tensors: the block's row is forced into [0, 2h), whole blocks)
+                            int64_t m = block_row - (int64_t)expert * (2 * p.out_half);
+                            m = m < 0 ? 0 : (m > 2 * p.out_half - 32 ? 2 * p.out_half - 32 : m);
+                            m &= ~(int64_t)31;
                             const bool upper = m >= p.out_half;
                             obase = (upper ? p.out2 : p.out) +
                                     ((int64_t)expert * p.out_half + (upper ? m - p.out_half : m)) * p.out_stride;
