@@ -278,7 +278,7 @@ def cpu_baseline(w, budget_s=12.0):
 
 def run_train(w, steps, warmup):
     """Forward + backward of the SwiGLU MoE through the differentiable operators (bf16): the
-    training step of SURVEY 8(f).1, reported beside the forward metric, never instead of it."""
+    training step, reported beside the forward metric, never instead of it."""
     from fast_moe_amd.kernels import moe
     from fast_moe_amd.kernels.hip import ops
     dev = torch.device("cuda:0")
@@ -312,7 +312,7 @@ def run_train(w, steps, warmup):
 
 
 def run_sgmoe(steps, warmup, tokens):
-    """The SGMoE layer with the MRN router front-end (SURVEY 8(f).3) at the 64-expert top-8 size of
+    """The SGMoE layer with the MRN router front-end at the 64-expert top-8 size of
     the headline workload (SiLU MLP experts, as the layer has them): evaluation forward,
     training step, and the share of the router front-end (norm, normalised-logit gating,
     dispatch) in the forward.  Reported beside the forward metric, never instead of it."""
