@@ -1462,13 +1462,21 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 constexpr bool LAST = decltype(last_c)::value;   // last of the tile: no fragments kept over the epilogue
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
                 const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
+                auto interleave = [&]() {   // one fragment read in the shadow of every MFMA
+#pragma unroll
+                    for (int i = 0; i < FM + FN; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, (WTR || XTR) ? 2 : 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN), 0);
+                };
                 load_block(wfb, xfb, cslot, 1, kitem, mask_c);
-                __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfa, xfa, std::false_type{});
+                interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 load_block(wfa, xfa, s1, 0, kitem + 1, mask_c);
-                __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfb, xfb, std::false_type{});
+                interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 barrier();                  // B
                 part_a = lds_base + islot * TL::STAGE_BYTES;    // pair (c+4, c+5)
@@ -1483,16 +1491,18 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 }
                 ikt += 2;
                 load_block(wfb, xfb, s1, 1, kitem + 1, mask_c);
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (HALF == 0) __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfa, xfa, std::integral_constant<bool, HALF == 0>{});
+                if constexpr (HALF != 0) interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 // pair (c+2, c+3) is older than the 2L instructions the first half just issued
                 if (HALF == 0) wait_vmcnt<2 * L>();
                 else wait_vmcnt<0>();
                 barrier();                  // A'
                 if (!LAST) load_block(wfa, xfa, s2, 0, kitem + 2, mask_c);
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (HALF == 1 || LAST) __builtin_amdgcn_sched_barrier(0);
                 mma_block(wfb, xfb, std::integral_constant<bool, HALF == 1>{});
+                if constexpr (HALF != 1 && !LAST) interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 cslot = s2;
                 kitem += 2;
