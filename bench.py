@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per GEMM1 launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
 # profiles/ (KiB per dispatch, scaled by the copy-kernel factors 2.0 and 1.0 stated there).
 MEASURED_TRAFFIC_BYTES = {
-    "c3_bf16": int((1.6404e6 * 2.0 + 3.6048e5 * 1.0) * 1024),
-    "c4_fp8": int((9.1855e5 * 2.0 + 3.649e5 * 1.0) * 1024),
+    "c3_bf16": int((1.6588e6 * 2.0 + 3.6049e5 * 1.0) * 1024),
+    "c4_fp8": int((9.0602e5 * 2.0 + 3.6486e5 * 1.0) * 1024),
 }
 
 WORKLOADS = {
