@@ -205,6 +205,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     auto run = [&](auto has_bias_c, auto has_aux_c) {
         constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
         constexpr bool HAS_AUX = SWIGLU && decltype(has_aux_c)::value;   // keep the pre-activations (training)
+        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && !FP8 && FN_OUT == 2;   // (the e4m3 kernels have no registers to spare for it)
         // per-column epilogue constants of this lane: [fn][gp][q][j] <-> column nq + 8*q + 4*khalf + j
         // with nq = first column of register-quad pair gp of fragment fn
         float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
@@ -242,6 +243,98 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         // rows outermost: the stores that complete a row's 128-byte line follow each other
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
+            if constexpr (QUAD) {
+                // The store unit merges what ADJACENT lanes write: a lane and its partner 32 lanes
+                // away cost two requests even for neighbouring bytes, four adjacent lanes on 64
+                // contiguous bytes cost one (a 128 KB tile drains in 1.3 us instead of 3.9).  So:
+                // the halves of the wave trade pieces until a low lane owns columns 0..31 of its row
+                // and its partner 32..63, then every quad of lanes transposes its 4 rows x 4 chunks
+                // of 16 bytes, and store i of the block writes row 4q + i from the 4 lanes of quad q.
+                uint32_t pk[8][2];          // piece g: columns 8g + 4*khalf + 0..3 of the wave's 64
+#pragma unroll
+                for (int fn = 0; fn < 2; ++fn)
+#pragma unroll
+                    for (int gp = 0; gp < 2; ++gp)
+#pragma unroll
+                        for (int q = 0; q < 2; ++q)
+#pragma unroll
+                            for (int j = 0; j < 4; j += 2) {
+                                const int v = 4 * (2 * gp + q) + j;
+                                float ya = acc[fn][fm][v], yb = acc[fn][fm][v + 1];
+                                if (FP8) {
+                                    ya *= rsa[fm] * rsw[fn][gp][q][j];
+                                    yb *= rsa[fm] * rsw[fn][gp][q][j + 1];
+                                    if (HAS_BIAS && p.bias) {
+                                        rbf2(ya, yb);
+                                        ya += bv[fn][gp][q][j];
+                                        yb += bv[fn][gp][q][j + 1];
+                                    }
+                                } else if (HAS_BIAS) {
+                                    ya += bv[fn][gp][q][j];
+                                    yb += bv[fn][gp][q][j + 1];
+                                }
+                                if (EPI == FMOE_EPI_SILU) {
+                                    rbf2(ya, yb);
+                                    ya = fast_silu_f32(ya);
+                                    yb = fast_silu_f32(yb);
+                                }
+                                pk[4 * fn + 2 * gp + q][j / 2] = pack_bf16(ya, yb);
+                            }
+                uint32_t ch[4][4];          // chunk c: columns 32*khalf + 8c + 0..7, afterwards row 4q + c's
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int d = 0; d < 2; ++d) {
+                        const u32x2 s = __builtin_amdgcn_permlane32_swap(pk[c][d], pk[c + 4][d], false, false);
+                        ch[c][d] = s[0];
+                        ch[c][2 + d] = s[1];
+                    }
+                int l = lane;
+                asm volatile("" : "+v"(l));
+                const bool odd = (l & 1) != 0, up = (l & 2) != 0;
+#pragma unroll
+                for (int pr = 0; pr < 4; pr += 2)       // lanes j, j ^ 1 trade across slots (pr, pr + 1)
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint32_t send = odd ? ch[pr][d] : ch[pr + 1][d];
+                        const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xF, 0xF, true);
+                        ch[pr][d] = odd ? recv : ch[pr][d];
+                        ch[pr + 1][d] = odd ? ch[pr + 1][d] : recv;
+                    }
+#pragma unroll
+                for (int pr = 0; pr < 2; ++pr)          // lanes j, j ^ 2 trade across slots (pr, pr + 2)
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint32_t send = up ? ch[pr][d] : ch[pr + 2][d];
+                        const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0x4E, 0xF, 0xF, true);
+                        ch[pr][d] = up ? recv : ch[pr][d];
+                        ch[pr + 2][d] = up ? ch[pr + 2][d] : recv;
+                    }
+                const int64_t block_row = row0 + wm * TM + fm * 32;
+                uint16_t* obase = p.out + block_row * p.out_stride;
+                if constexpr (OUT2) {
+                    if (p.out2) {       // (as below: wave-uniform, forced into the two tensors)
+                        int64_t m = block_row - (int64_t)expert * (2 * p.out_half);
+                        m = m < 0 ? 0 : (m > 2 * p.out_half - 32 ? 2 * p.out_half - 32 : m);
+                        m &= ~(int64_t)31;
+                        const bool upper = m >= p.out_half;
+                        obase = (upper ? p.out2 : p.out) +
+                                ((int64_t)expert * p.out_half + (upper ? m - p.out_half : m)) * p.out_stride;
+                    }
+                }
+                const int quad_row = 4 * ((l & 31) >> 2);
+                const int col = col0 + 32 * (l >> 5) + 8 * (l & 3);
+                const uint32_t lane_off = ((uint32_t)quad_row * (uint32_t)p.out_stride + (uint32_t)(32 * (l >> 5) + 8 * (l & 3))) * 2u;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uint16_t* base = obase + i * p.out_stride + col0;
+                    if (wm * TM + fm * 32 + quad_row + i < rows_valid && col + 7 < p.N)
+                        *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(base) + lane_off) =
+                            u32x4{ch[i][0], ch[i][1], ch[i][2], ch[i][3]};
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                continue;
+            }
 #pragma unroll
             for (int fn = 0; fn < FN_OUT; ++fn) {
 #pragma unroll
