@@ -128,6 +128,7 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
                   (!d->aux || ((d->aux_stride_row % vec_cols == 0) && aligned16(d->aux) && aligned16(d->aux2) &&
                                d->aux_stride_row < stride_cap));
 
+    p.scale_vec = fp8 && d->n >= 4 && d->n % 4 == 0 && aligned16(d->b_scale) && (!d->b2_scale || aligned16(d->b2_scale));
     const int esize = fp8 ? 1 : (f32 ? 4 : 2);
     const int chunk = 16 / esize;
     const bool fast = d->b_stride_k == 1 && (d->k % chunk) == 0 && aligned16(d->a) && aligned16(d->b) &&

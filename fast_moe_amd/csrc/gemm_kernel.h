@@ -65,6 +65,7 @@ struct GemmParams {
     int64_t out_stride;
     int n_tiles;
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
+    int scale_vec;                      // e4m3: 16-byte loads of 4 weight scales are legal
     const int64_t* k_window;            // [E+1] per-expert contraction range, or null
     int k_window_multiple;              // every window is a multiple of this and at least twice it (0: unknown)
     uint16_t* aux;                      // SWIGLU: the two pre-activations, or null
@@ -227,9 +228,11 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
                         const int nc = n < p.N ? n : p.N - 1;
                         // (v_rcp_f32 is exact on the powers of two the reference's scales are)
-                        rsw[fn][gp][q][j] = FP8 ? __builtin_amdgcn_rcpf(p.b_scale[(int64_t)expert * p.N + nc]) : 1.0f;
-                        rsw2[fn][gp][q][j] =
-                            (FP8 && SWIGLU) ? __builtin_amdgcn_rcpf(p.b2_scale[(int64_t)expert * p.N + nc]) : 1.0f;
+                        rsw[fn][gp][q][j] = rsw2[fn][gp][q][j] = 1.0f;
+                        if (FP8 && !p.scale_vec) {
+                            rsw[fn][gp][q][j] = __builtin_amdgcn_rcpf(p.b_scale[(int64_t)expert * p.N + nc]);
+                            if (SWIGLU) rsw2[fn][gp][q][j] = __builtin_amdgcn_rcpf(p.b2_scale[(int64_t)expert * p.N + nc]);
+                        }
                         bv[fn][gp][q][j] = bv2[fn][gp][q][j] = 0.0f;
                         if (HAS_BIAS) {
                             const float a = bf16_bits_to_f32(bias_a[bias_row + nc]);
@@ -240,6 +243,28 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                             bv2[fn][gp][q][j] = p.bias2 ? b : 0.0f;
                         }
                     }
+        if (FP8 && p.scale_vec) {
+            // the 4 scales of a register quad in one 16-byte load (a quad that begins past the
+            // last column reads the last 4 scales instead: its columns are never stored)
+#pragma unroll
+            for (int fn = 0; fn < FN_OUT; ++fn)
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp)
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf;
+                        const int64_t at = (int64_t)expert * p.N + (n + 3 < p.N ? n : p.N - 4);
+                        typedef __attribute__((ext_vector_type(4))) float f32x4;
+                        const f32x4 s1 = *reinterpret_cast<const f32x4*>(p.b_scale + at);
+                        f32x4 s2 = s1;
+                        if (SWIGLU) s2 = *reinterpret_cast<const f32x4*>(p.b2_scale + at);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            rsw[fn][gp][q][j] = __builtin_amdgcn_rcpf(s1[j]);
+                            if (SWIGLU) rsw2[fn][gp][q][j] = __builtin_amdgcn_rcpf(s2[j]);
+                        }
+                    }
+        }
         __builtin_amdgcn_sched_barrier(0);
         // rows outermost: the stores that complete a row's 128-byte line follow each other
 #pragma unroll

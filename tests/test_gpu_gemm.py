@@ -689,3 +689,36 @@ def test_silu_jagged_bmm_fp8(lens, Din, Dout):
     raw = torch.cat([torch.nn.functional.silu(j[offsets[e]:offsets[e + 1]].float()) @ w[e].float().T + b[e].float()
                      for e in range(E)])
     assert (out.float().cpu() - raw).abs().max().item() <= 0.1 * scale
+
+
+@pytest.mark.parametrize("swiglu", [False, True])
+@pytest.mark.parametrize("M", [96, 8192])
+def test_fp8_weight_scales_at_any_alignment(M, swiglu):
+    """The e4m3 epilogue loads a register quad's 4 weight scales at once when the scale tensors sit
+    on 16-byte boundaries and one by one otherwise: both give the same bits."""
+    from fast_moe_amd.kernels.hip import ops
+    E, K, N = 8, 512, 512
+    g = torch.Generator().manual_seed(77 + M)
+    a = torch.randn(M, K, generator=g).to(BF16).cuda()
+    w = [torch.randn(E * N, K, generator=g).to(BF16).cuda() for _ in range(2)]
+    offsets = (torch.arange(E + 1, dtype=torch.int64) * (M // E)).cuda()
+    qa, sa = ops.quant_rows_fp8(a)
+    (qb, sb), (qb2, sb2) = ops.quant_rows_fp8(w[0]), ops.quant_rows_fp8(w[1])
+    # make the scales differ from column to column by more than the quantiser's choice does
+    sb = sb * torch.tensor([1.0, 2.0, 0.5, 4.0], device="cuda").repeat(E * N // 4)
+    sb2 = sb2 * torch.tensor([0.25, 1.0, 8.0, 2.0], device="cuda").repeat(E * N // 4)
+
+    def run(shift):
+        def place(s):
+            buf = torch.zeros(E * N + 4, device="cuda")
+            buf[shift:shift + E * N] = s
+            return buf[shift:shift + E * N].view(E, N)
+        kw = dict(total_rows=M, a_scale=sa, b_scale=place(sb))
+        if swiglu:
+            kw.update(b2=qb2.view(E, N, K).permute(0, 2, 1), b2_scale=place(sb2), epilogue=ops.EPI_SWIGLU)
+        return ops.grouped_gemm(offsets, qa, qb.view(E, N, K).permute(0, 2, 1), **kw)
+
+    aligned = run(0)
+    assert aligned.float().abs().max() > 0
+    for shift in (1, 2, 3):
+        assert torch.equal(run(shift), aligned)
