@@ -183,7 +183,8 @@ typedef struct fmoe_gemm_desc {
     const void* b;          /* same dtype as A                                    */
     const void* b2;         /* second weight (SWIGLU) or NULL                     */
     int64_t b_stride_e, b_stride_k, b_stride_n;
-    const float* b_scale;   /* [E, n] multiplier scales (FMOE_E4M3)               */
+    const float* b_scale;   /* [E, n] multiplier scales (FMOE_E4M3); any 4-byte
+                             * alignment works, 16-byte alignment loads 4 at a time */
     const float* b2_scale;
 
     const void* bias;       /* [E, n] in out_dtype, or NULL                       */
