@@ -722,3 +722,36 @@ def test_fp8_weight_scales_at_any_alignment(M, swiglu):
     assert aligned.float().abs().max() > 0
     for shift in (1, 2, 3):
         assert torch.equal(run(shift), aligned)
+
+
+@pytest.mark.parametrize("epi", ["none", "silu", "swiglu"])
+@pytest.mark.parametrize("M", [96, 8192])
+def test_bias_at_any_alignment(M, epi):
+    """Bias tensors at any 2-byte alignment and with any expert pitch give the same bits."""
+    from fast_moe_amd.kernels.hip import ops
+    E, K, N = 8, 256, 512
+    g = torch.Generator().manual_seed(5 + M)
+    a = torch.randn(M, K, generator=g).to(BF16).cuda()
+    w = [(torch.randn(E, K, N, generator=g) / 16).to(BF16).cuda() for _ in range(2)]
+    bias = [torch.randn(E, N, generator=g).to(BF16).cuda() for _ in range(2)]
+    offsets = (torch.arange(E + 1, dtype=torch.int64) * (M // E)).cuda()
+
+    def run(shift, pitch):
+        def place(b):
+            buf = torch.zeros(E * pitch + 8, dtype=BF16, device="cuda")
+            v = buf[shift:shift + E * pitch].view(E, pitch)[:, :N]
+            v.copy_(b)
+            return v
+        kw = dict(total_rows=M, bias=place(bias[0]))
+        if epi == "swiglu":
+            kw.update(b2=w[1], bias2=place(bias[1]), epilogue=ops.EPI_SWIGLU)
+        elif epi == "silu":
+            kw.update(epilogue=ops.EPI_SILU)
+        return ops.grouped_gemm(offsets, a, w[0], **kw)
+
+    aligned = run(0, N)
+    ref = a[:M // E].float() @ w[0][0].float() + bias[0][0].float()
+    if epi == "none":
+        torch.testing.assert_close(aligned[:M // E].float(), ref.to(BF16).float(), atol=3e-2, rtol=1.6e-2)
+    for shift, pitch in ((1, N), (2, N), (3, N), (0, N + 2), (4, N + 4)):
+        assert torch.equal(run(shift, pitch), aligned), (shift, pitch)
