@@ -62,8 +62,18 @@ __device__ __forceinline__ void store_score<float>(float* p, float v) { *p = v; 
 template <>
 __device__ __forceinline__ void store_score<uint16_t>(uint16_t* p, float v) { *p = (uint16_t)f32_to_bf16_bits(v); }
 
+// Total order on scores as unsigned keys: NaN above +inf (where torch.topk and torch.sort put
+// it), -0 equal to +0, otherwise the order of the values.  With keys every token fills exactly K
+// distinct slots whatever its scores hold; a float comparison ranks every NaN first at once.
+__device__ __forceinline__ uint32_t order_key(float v) {
+    const uint32_t b = __float_as_uint(v);
+    if ((b & 0x7FFFFFFFu) > 0x7F800000u) return 0xFFFFFFFFu;     // NaN
+    if ((b & 0x7FFFFFFFu) == 0u) return 0x80000000u;             // +-0
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
 // One token per LPT lanes, VPL scores per lane (expert id = v*LPT + sub).  The
-// rank of a score is the number of scores that beat it (greater, or equal with
+// rank of a score is the number of scores that beat it (greater key, or equal key with
 // a lower expert id); rank < K selects it and is its slot.
 template <typename T, int LPT, int VPL>
 __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores, int64_t num_tokens,
@@ -108,21 +118,24 @@ __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores,
         }
     }
     int rank[VPL];
+    uint32_t key[VPL];
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) rank[v] = 0;
+    for (int v = 0; v < VPL; ++v) {
+        rank[v] = 0;
+        key[v] = order_key(my[v]);
+    }
 #pragma unroll
     for (int u = 0; u < VPL; ++u) {
 #pragma unroll
         for (int i = 0; i < LPT; ++i) {
             // a full wave per token: the broadcast lane is a compile-time constant (v_readlane)
-            const float other = LPT == kWave
-                                    ? __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(my[u]), i))
-                                    : __shfl(my[u], grp * LPT + i, kWave);
+            const uint32_t other = LPT == kWave ? (uint32_t)__builtin_amdgcn_readlane((int)key[u], i)
+                                                : (uint32_t)__shfl((int)key[u], grp * LPT + i, kWave);
             const int oe = u * LPT + i;
 #pragma unroll
             for (int v = 0; v < VPL; ++v) {
                 const int e = v * LPT + sub;
-                rank[v] += (other > my[v] || (other == my[v] && oe < e)) ? 1 : 0;
+                rank[v] += (other > key[v] || (other == key[v] && oe < e)) ? 1 : 0;
             }
         }
     }
@@ -151,7 +164,8 @@ __global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores,
     if (renorm == 1) {
         float s = 0.0f;
         for (int j = 0; j < K; ++j) s = s + fabsf(s_sel[wave][grp][j]);   // slot order
-        denom = fmaxf(round_to<T>(s), round_to<T>(1e-12f));
+        // (clamp_min keeps a NaN norm, fmaxf would drop it)
+        denom = s != s ? s : fmaxf(round_to<T>(s), round_to<T>(1e-12f));
     }
     float nmax = 0.0f;
     if (renorm >= 2) {

@@ -249,11 +249,13 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  b2_scale: Optional[torch.Tensor] = None, a_expert_stride: int = 0,
                  k_window: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                  k_window_multiple: int = 0,
-                 aux: Optional[Tuple[torch.Tensor, torch.Tensor]] = None) -> torch.Tensor:
+                 aux: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                 plan_only: bool = False) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
     strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
     [total_rows, N] in bf16 (fp32 for fp32 operands).  ``aux`` = two tensors like the output
-    that receive the SWIGLU pre-activations."""
+    that receive the SWIGLU pre-activations.  ``plan_only``: launch nothing and return the
+    _lib.PLAN_* code of the kernel this call would run (fmoe_grouped_gemm_plan)."""
     dev = _need_cuda("grouped_gemm", offsets, a, b, row_index, bias, b2, bias2, a_scale, b_scale, b2_scale)
     fp8 = a.dtype == FP8_DTYPE
     if not fp8 and a.dtype not in (torch.bfloat16, torch.float32):
@@ -297,7 +299,7 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                 raise ValueError(f"grouped_gemm: aux tensors must be {out_dtype} [{total_rows}, {N}] with "
                                  "contiguous rows and one row stride")
     if total_rows == 0:
-        return out
+        return _lib.PLAN_NONE if plan_only else out
 
     def bias_ok(t):
         if t is None:
@@ -369,6 +371,8 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
             d.a, d.a_stride_row = a.data_ptr(), a.stride(0)
         else:
             d.a_silu = 1
+    if plan_only:
+        return gemm_plan(d)
     rc = lib.fmoe_grouped_gemm(ctypes.byref(d), _stream(a))
     _lib.check(rc, "fmoe_grouped_gemm")
     return out

@@ -41,15 +41,21 @@ def quantize_expert_weights(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.T
 
 
 class _WeightQuantCache:
-    """(fp8 bytes, scales) of expert weights, kept until the weight changes.
+    """(fp8 bytes, scales) of expert weights, kept until the weight changes.  OPT-IN: the
+    operators below quantise their weight on every call, as the reference does
+    (kernels/pytorch/moe_fp8.py:111, kernels/triton/triton_moe_fp8.py:1157, 1423: 3 bytes of
+    HBM traffic per weight element per forward); a caller that wants to pay that once per weight
+    update passes ``fp8_weight=cached_quantize_expert_weights(w)`` (or its own pair).
 
-    The reference quantises the weights inside every fp8 operator call
-    (kernels/pytorch/moe_fp8.py:111, kernels/triton/triton_moe_fp8.py:1157, 1423): 3 bytes of
-    HBM traffic per weight element per forward.  An entry is keyed by the tensor that owns
-    the storage (the parameter behind a ``permute``/``to`` view, held weakly) and by the
-    view's geometry; it is dropped when the owner's in-place version counter moves (an
-    optimizer step, ``copy_``, ``load_state_dict``) or the owner dies.  Out-of-place
-    replacement (``layer.w = new``) makes a new owner and therefore a new entry.
+    An entry is keyed by the tensor that owns the storage (the parameter behind a
+    ``permute``/``to`` view, held weakly) and by the view's geometry; it is dropped when the
+    owner's in-place version counter moves (an optimizer step, ``copy_``, ``load_state_dict``)
+    or the owner dies; dead owners are purged on every insert.  Out-of-place replacement
+    (``layer.w = new``) makes a new owner and therefore a new entry.
+
+    What the version counter does NOT see: writes through ``param.data`` (``p.data.mul_()``,
+    hand-written optimizers, EMA updates, flat-parameter swaps that keep the pointer).  After
+    such a write call ``invalidate(weight)`` (or ``clear()``), or do not use the cache.
     """
 
     def __init__(self, max_entries: int = 32) -> None:
@@ -74,12 +80,18 @@ class _WeightQuantCache:
                 return value
         self.misses += 1
         value = quantize(weight)
-        if len(self._entries) >= self._max:
-            dead = [k for k, (r, *_rest) in self._entries.items() if r() is None]
-            for k in dead or list(self._entries)[:1]:
-                self._entries.pop(k, None)
+        for k in [k for k, (r, *_rest) in self._entries.items() if r() is None]:
+            self._entries.pop(k, None)
+        self._entries.pop(key, None)
+        while len(self._entries) >= self._max:
+            self._entries.pop(next(iter(self._entries)))
         self._entries[key] = (weakref.ref(owner), owner._version, geom, value)
         return value
+
+    def invalidate(self, weight: torch.Tensor) -> None:
+        """Drop the entry of the tensor that owns ``weight``'s storage (after a write the
+        version counter cannot see)."""
+        self._entries.pop(id(self._owner(weight)), None)
 
     def clear(self) -> None:
         self._entries.clear()
@@ -89,8 +101,22 @@ weight_quant_cache = _WeightQuantCache()
 
 
 def cached_quantize_expert_weights(weight: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """``quantize_expert_weights`` through ``weight_quant_cache``."""
+    """``quantize_expert_weights`` through ``weight_quant_cache`` (see its caveat on ``.data``
+    writes); the result is what the operators take as ``fp8_weight``."""
     return weight_quant_cache.get(weight, quantize_expert_weights)
+
+
+def _weight_pair(weight: torch.Tensor, fp8_weight) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The (e4m3 [E, K, N], scale [E, N]) pair of ``weight``: the caller's, checked for shape, or a
+    fresh quantisation."""
+    if fp8_weight is None:
+        return quantize_expert_weights(weight)
+    q, s = fp8_weight
+    if (q.dtype != ops.FP8_DTYPE or tuple(q.shape) != tuple(weight.shape) or s.dtype != torch.float32
+            or tuple(s.shape) != (weight.shape[0], weight.shape[2]) or q.device != weight.device):
+        raise ValueError(f"fp8_weight must be (float8_e4m3fn {tuple(weight.shape)}, fp32 "
+                         f"{(weight.shape[0], weight.shape[2])}) on {weight.device}")
+    return q, s
 
 
 def silu_jagged_fp8(
@@ -125,13 +151,16 @@ def silu_jagged_bmm_fp8(
     weight: torch.Tensor,
     bias: torch.Tensor,
     kernel: KernelType = KernelType.HIP,
+    *,
+    fp8_weight: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> torch.Tensor:
     """kernels/moe_fp8.py:98-124 with weight [E, D_out, D_in] (kernels/pytorch/moe_fp8.py:46-75):
-    ``silu(jagged)`` row-quantised, weight row-quantised, fp8 GEMM + bias."""
+    ``silu(jagged)`` row-quantised, weight row-quantised, fp8 GEMM + bias.  ``fp8_weight``: the
+    pair ``quantize_expert_weights(weight.permute(0, 2, 1))`` when the caller keeps it."""
     require_hip_kernel(kernel, "silu_jagged_bmm_fp8")
     ops._forward_only("silu_jagged_bmm_fp8", jagged, weight, bias)
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=True)
-    qw, sw = cached_quantize_expert_weights(weight.permute(0, 2, 1))    # rows of [E, D_out, D_in], once per update
+    qw, sw = _weight_pair(weight.permute(0, 2, 1), fp8_weight)          # rows of [E, D_out, D_in]
     return ops.grouped_gemm(seq_offsets, qa, qw, total_rows=jagged.shape[0], bias=bias,
                             a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
 
@@ -149,13 +178,16 @@ def silu_jagged_bmm_combine_fp8(
     activation_checkpointing: bool = False,
     has_silu: bool = True,
     kernel: KernelType = KernelType.HIP,
+    *,
+    fp8_weight: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> torch.Tensor:
     """kernels/moe_fp8.py:127-182: (SiLU +) row-quant of the hidden, weight row-quant, fp8 grouped
-    GEMM + bias, weighted merge.  weight is [E, D_in, D_out]."""
+    GEMM + bias, weighted merge.  weight is [E, D_in, D_out]; it is quantised on every call unless
+    ``fp8_weight = quantize_expert_weights(weight)`` is handed in."""
     require_hip_kernel(kernel, "silu_jagged_bmm_combine_fp8")
     L, K = reverse_index.shape
     assert index.shape[0] == L * K == jagged.shape[0]
-    qw, sw = cached_quantize_expert_weights(weight)
+    qw, sw = _weight_pair(weight, fp8_weight)
     if _ag.needs_grad(jagged, weight, bias, gating_scores):   # forward in e4m3, backward in bf16
         return _ag.SiluJaggedBmmCombine.apply(offsets, jagged, weight, bias, index, reverse_index, gating_scores,
                                               gates_index, has_silu, (qw, sw), activation_checkpointing)
@@ -174,10 +206,13 @@ def index_select_jagged_bmm(
     bias: Optional[torch.Tensor],
     kernel: KernelType = KernelType.HIP,
     fp8: bool = False,
+    *,
+    fp8_weight: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> torch.Tensor:
     """kernels/moe_fp8.py:185-248.  fp8=True: tokens quantised per row BEFORE the gather, weight
     per output row, fp8 MFMA GEMM, ``acc / (s_a x s_w)`` cast to bf16, plus bias
-    (kernels/pytorch/moe_fp8.py:98-139).  fp8=False: the bf16 operator."""
+    (kernels/pytorch/moe_fp8.py:98-139); the weight is quantised on every call, as there, unless
+    ``fp8_weight = quantize_expert_weights(weight)`` is handed in.  fp8=False: the bf16 operator."""
     require_hip_kernel(kernel, "index_select_jagged_bmm")
     assert index.ndim == 2 and index.shape[0] == jagged.shape[0]
     if not fp8:
@@ -186,7 +221,7 @@ def index_select_jagged_bmm(
         return ops.grouped_gemm(offsets, jagged, weight, total_rows=index.numel(), row_index=index,
                                 index_div=index.shape[-1], bias=bias, epilogue=EPI_NONE)
     assert jagged.dtype == weight.dtype and (bias is None or jagged.dtype == bias.dtype)
-    qw, sw = cached_quantize_expert_weights(weight)
+    qw, sw = _weight_pair(weight, fp8_weight)
     if _ag.needs_grad(jagged, weight, bias):
         return _ag.IndexSelectJaggedBmmFp8.apply(offsets, index, jagged, weight, bias, (qw, sw))
     qa, sa = ops.quant_rows_fp8(jagged)

@@ -72,12 +72,17 @@ class FastMoELayer(nn.Module):
         scores = self.gate(x).reshape(-1, self.num_experts)
         return ops.route_topk(scores, num_experts_per_tok, renorm=True)
 
-    def quantized_expert_weights(self) -> Dict[str, torch.Tensor]:
+    def quantized_expert_weights(self, refresh: bool = False) -> Dict[str, torch.Tensor]:
         """Row-quantised e4m3 copies of both expert weight tensors in the layout the fp8 operators
-        take ([E, D_in, D_out] views of K-contiguous bytes) with their [E, D_out] multiplier scales.
-        Kept beside the parameters (not in the state_dict) until a parameter is updated in place
-        or replaced; the reference re-quantises on every call (kernels/pytorch/moe_fp8.py:111)."""
-        from ..kernels.moe_fp8 import cached_quantize_expert_weights
+        take as ``fp8_weight`` ([E, D_in, D_out] views of K-contiguous bytes) with their [E, D_out]
+        multiplier scales.  Kept beside the parameters (not in the state_dict) until a parameter
+        is updated in place or replaced; the reference re-quantises on every call
+        (kernels/pytorch/moe_fp8.py:111).  Writes through ``param.data`` do not move the version
+        counter the cache watches: pass ``refresh=True`` after such an update."""
+        from ..kernels.moe_fp8 import cached_quantize_expert_weights, weight_quant_cache
+        if refresh:
+            weight_quant_cache.invalidate(self._experts_hidden_w)
+            weight_quant_cache.invalidate(self._experts_w)
         qh, sh = cached_quantize_expert_weights(self._experts_hidden_w.permute(0, 2, 1))
         qo, so = cached_quantize_expert_weights(self._experts_w.permute(0, 2, 1))
         return {"hidden_w": qh, "hidden_scale": sh, "out_w": qo, "out_scale": so}

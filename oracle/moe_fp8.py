@@ -24,15 +24,63 @@ def _dtype_name(t: torch.Tensor) -> str:
     return {torch.bfloat16: "bf16", torch.float32: "fp32"}[t.dtype]
 
 
-def rowwise_quant_fp8(a: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
-    """quant_fp8.py:27-34 on a torch tensor: returns (uint8 codes, fp32 multiplier scale)."""
-    codes, scale = _fp8.rowwise_quant_fp8(a.contiguous().float().numpy(), _dtype_name(a))
-    return torch.from_numpy(codes), torch.from_numpy(scale)
+# rows x cols above which rowwise_quant_fp8 takes the library cast instead of the bit-level encoder
+_BITS_LIMIT = 1 << 21
+
+
+def rowwise_quant_fp8(a: torch.Tensor, cast: Optional[str] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """quant_fp8.py:27-34 on a torch tensor: returns (uint8 codes, fp32 multiplier scale).
+
+    ``cast="bits"``: the numpy bit-level encoder of oracle.fp8 (about 1 us per element).
+    ``cast="torch"``: the same scale formula, then ``Tensor.to(torch.float8_e4m3fn)``, the
+    library routine quant_fp8.py:33 itself calls; for the operands of the large configurations
+    (10^9 weight elements).  Default: by size.  tests/test_oracle_fp8.py pins the two against
+    each other (random rows, outliers, zeros, subnormal results, inf / NaN rows)."""
+    if cast is None:
+        cast = "bits" if a.numel() <= _BITS_LIMIT else "torch"
+    if cast == "bits":
+        codes, scale = _fp8.rowwise_quant_fp8(a.contiguous().float().numpy(), _dtype_name(a))
+        return torch.from_numpy(codes), torch.from_numpy(scale)
+    assert cast == "torch", cast
+    amax = a.abs().amax(dim=-1).float()
+    scale = torch.from_numpy(_fp8.calculate_scale(amax.numpy(), _dtype_name(a)))
+    codes = torch.empty(a.shape, dtype=torch.uint8)
+    flat_a, flat_c, flat_s = a.reshape(-1, a.shape[-1]), codes.view(-1, a.shape[-1]), scale.reshape(-1)
+    step = max(1, (1 << 24) // a.shape[-1])         # bounded fp32 temporaries
+    for lo in range(0, flat_a.shape[0], step):
+        scaled = flat_a[lo: lo + step].float() * flat_s[lo: lo + step, None]
+        flat_c[lo: lo + step] = scaled.to(torch.float8_e4m3fn).view(torch.uint8)
+    return codes, scale
 
 
 def dequant(codes: torch.Tensor) -> torch.Tensor:
-    """uint8 e4m3fn codes -> fp32 values."""
+    """uint8 e4m3fn codes -> fp32 values (large operands: the library's decode, equal to the
+    table of oracle.fp8 for all 256 codes by tests/test_oracle_fp8.py)."""
+    if codes.numel() > _BITS_LIMIT:
+        return codes.contiguous().view(torch.float8_e4m3fn).to(torch.float32)
     return torch.from_numpy(_fp8.e4m3fn_decode(codes.numpy()))
+
+
+class LazyDequant:
+    """``q_w[e]`` -> fp32 values [N, K] of expert e's e4m3 codes, decoded on demand: the weight
+    operand of ``fp8_linear_per_expert`` for configurations whose decoded weights would not be
+    worth holding (10^9 elements)."""
+
+    def __init__(self, codes: torch.Tensor):
+        self.codes = codes
+
+    def __getitem__(self, e):
+        return dequant(self.codes[e])
+
+    def __len__(self):
+        return self.codes.shape[0]
+
+
+def quantize_weight(w: torch.Tensor):
+    """Weight [E, K, N] (any strides) -> (LazyDequant over codes [E, N, K], scale [E, N]): one scale
+    per (expert, output row), the quantisation moe_fp8.py:111 applies to ``weight.permute(0, 2, 1)``."""
+    codes, scale = rowwise_quant_fp8(w.permute(0, 2, 1))
+    return LazyDequant(codes), scale
 
 
 def index_select_jagged_bmm_raw(offsets, index, jagged, weight, bias):
@@ -59,6 +107,9 @@ def fp8_linear_per_expert(q_rows: List[torch.Tensor], s_rows: List[torch.Tensor]
     """
     out = []
     for e in range(len(q_rows)):
+        if q_rows[e].shape[0] == 0:                 # an expert without rows: nothing to decode
+            out.append(torch.empty((0, s_w.shape[1]), dtype=out_dtype))
+            continue
         acc = torch.matmul(q_rows[e].to(torch.bfloat16), q_w[e].T.to(torch.bfloat16))
         y = (acc / (s_rows[e][:, None] * s_w[e][None, :])).to(out_dtype)
         out.append(y + (bias[e] if bias is not None else 0))
@@ -127,12 +178,14 @@ def index_select_jagged_bmm_fp8_backward(offsets, index, jagged, weight, bias, d
 
 
 def swiglu_moe_fp8(offsets, index, jagged, w_gate, b_gate, w_up, b_up, w_down, b_down,
-                   token_index, k, gates=None, gates_index=None):
+                   token_index, k, gates=None, gates_index=None, quantized=None):
     """The fp8 SwiGLU MoE forward as a composition of the emulated fp8 GEMM:
     tokens quantised per row before the gather, gate/up weights per output row,
     ``silu(g) * u`` with the bf16 rounding points of moe.py:125-139, hidden
     re-quantised per row, down projection, weighted merge (moe.py:14-37).
-    Weights are given [E, K, N] like every operator.  Returns (out, hidden)."""
+    Weights are given [E, K, N] like every operator.  ``quantized``: the three
+    ``quantize_weight`` results of (w_gate, w_up, w_down) when the caller holds them already
+    (then the weight arguments are not read).  Returns (out, hidden)."""
     dt = jagged.dtype
     qa_c, s_a = rowwise_quant_fp8(jagged)
     q_a = dequant(qa_c)
@@ -141,19 +194,15 @@ def swiglu_moe_fp8(offsets, index, jagged, w_gate, b_gate, w_up, b_up, w_down, b
     q_rows = list(q_a[token].split(sizes))
     s_rows = list(s_a[token].split(sizes))
 
-    def w_quant(w):
-        c, s = rowwise_quant_fp8(w.permute(0, 2, 1))
-        return dequant(c), s
-
-    qg, sg = w_quant(w_gate)
-    qu, su = w_quant(w_up)
+    if quantized is None:
+        quantized = (quantize_weight(w_gate), quantize_weight(w_up), quantize_weight(w_down))
+    (qg, sg), (qu, su), (qd, sd) = quantized
     g = fp8_linear_per_expert(q_rows, s_rows, qg, sg, b_gate, dt)
     u = fp8_linear_per_expert(q_rows, s_rows, qu, su, b_up, dt)
     hidden = torch.cat([F.silu(x) * y for x, y in zip(g, u)], dim=0)
 
     qh_c, s_h = rowwise_quant_fp8(hidden)
     q_h = dequant(qh_c)
-    qd, sd = w_quant(w_down)
     y = torch.cat(
         fp8_linear_per_expert(list(q_h.split(sizes)), list(s_h.split(sizes)), qd, sd, b_down, dt),
         dim=0,

@@ -56,6 +56,17 @@ def complete_cumsum(lengths: np.ndarray) -> np.ndarray:
     return out
 
 
+def order_key(scores: np.ndarray) -> np.ndarray:
+    """int64 key whose order is the order torch.topk ranks float32 scores by: increasing value,
+    -0 == +0, every NaN equal and above +inf."""
+    scores = np.ascontiguousarray(scores, dtype=np.float32)
+    bits = scores.view(np.uint32).astype(np.int64)
+    mag = bits & 0x7FFFFFFF
+    key = np.where(bits & 0x80000000 != 0, 0x7FFFFFFF - mag, 0x80000000 + mag)
+    key = np.where(mag == 0, 0x80000000, key)
+    return np.where(mag > 0x7F800000, 0xFFFFFFFF, key)
+
+
 def select_top_k(scores: np.ndarray, k: int, dtype: str = "fp32", renorm: bool = True):
     """Canonical top-k + L1 renormalisation (fast_moe_module.py:93-105).
 
@@ -71,8 +82,9 @@ def select_top_k(scores: np.ndarray, k: int, dtype: str = "fp32", renorm: bool =
     scores = np.asarray(scores, dtype=np.float32)
     T, E = scores.shape
     assert 1 <= k <= E
-    # stable argsort of the negated scores: descending value, ties -> lower index
-    order = np.argsort(-scores, axis=1, kind="stable")[:, :k].astype(np.int64)
+    # stable descending sort on a total order: NaN above +inf (torch.topk / torch.sort treat NaN as
+    # the largest value), -0 equal to +0, ties -> lower index
+    order = np.argsort(-order_key(scores), axis=1, kind="stable")[:, :k].astype(np.int64)
     vals = np.take_along_axis(scores, order, axis=1)
     if not renorm:
         return order, vals
@@ -80,7 +92,8 @@ def select_top_k(scores: np.ndarray, k: int, dtype: str = "fp32", renorm: bool =
     for j in range(k):  # sequential fp32 accumulation in slot order
         s = (s + np.abs(vals[:, j])).astype(np.float32)
     denom = np.maximum(_round(s, dtype), _round(np.float32(_EPS), dtype)).astype(np.float32)
-    gates = _round((vals / denom[:, None]).astype(np.float32), dtype)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        gates = _round((vals / denom[:, None]).astype(np.float32), dtype)
     return order, gates
 
 

@@ -1,0 +1,298 @@
+"""The SwiGLU MoE chain (route -> gather + GEMM1 + SwiGLU -> [row quant] -> GEMM2 -> merge) on the
+GPU through the operator wrappers, and stage-by-stage oracle checks on sampled rows / tokens.
+
+Shared by the full-size parity tests.  A stage is checked twice where that is possible:
+* on the GPU's own inputs of that stage (copied to the CPU), element by element within a few
+  bf16 ulps plus the fp32-accumulation floor -- this isolates the kernel of the stage;
+* end to end against the oracle's own chain at the tolerance the baseline states.
+"""
+import numpy as np
+import torch
+from torch.nn import functional as F
+
+from oracle import moe as o_moe
+from oracle import moe_fp8 as o_fp8
+from oracle import routing as o_routing
+
+BF16 = torch.bfloat16
+# Absolute error floors as fractions of S = sum_k |a_k| |b_k| (the scale of a dot product's rounding
+# error), for entries that are small by cancellation.  Measured on MI355X against float64 on
+# 1536-term sums: bf16 operands (exact products, fp32 accumulation in some order) up to 2^-20.6 of
+# S; e4m3 operands up to 2^-18.3 of S on random data and 2^-16.3 of S over the 2 * 10^6 outputs
+# of the 128-expert configuration (the MFMA adds the 64 products of one instruction in a
+# block-aligned adder that keeps fewer bits than an fp32 sum).  The floors leave a factor 4.
+BF16_FLOOR = 2.0 ** -18
+FP8_FLOOR = 2.0 ** -14
+
+
+# ------------------------------------------------------------------ comparisons
+def bf16_ulp(ref):
+    """Spacing of bf16 numbers at |ref| (0 at 0)."""
+    a = ref.float().abs()
+    _, e = torch.frexp(a)
+    ulp = torch.ldexp(torch.ones_like(a), e - 8)
+    return torch.where(a == 0, torch.zeros_like(a), ulp)
+
+
+def assert_ulp_close(got, ref, ulps, floor, what):
+    """|got - ref| <= ulps * ulp_bf16(ref) + floor, element by element.  `floor` (tensor or number)
+    is the absolute error an fp32 accumulation in another order may leave, so that entries that
+    are small by cancellation are not held to a relative bound that no summation order meets."""
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    err = (got - ref).abs()
+    bound = ulps * bf16_ulp(ref) + floor
+    bad = ~(err <= bound)
+    if bad.any():
+        i = int(torch.argmax((err - bound).flatten()))
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.numel()} elements beyond {ulps} bf16 ulps; worst "
+                             f"err {err.flatten()[i].item():.4g} at ref {ref.flatten()[i].item():.4g}")
+
+
+def assert_within(got, ref, bound, what):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    err = (got - ref).abs()
+    bad = ~(err <= bound)
+    if bad.any():
+        i = int(torch.argmax((err - bound).flatten()))
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.numel()} elements out of bound; worst err "
+                             f"{err.flatten()[i].item():.4g} (bound {bound.flatten()[i].item():.4g}) at ref "
+                             f"{ref.flatten()[i].item():.4g}")
+
+
+def swiglu_ref_and_bound(g_ref, u_ref, floor_g, floor_u):
+    """h = silu(g) * u from the oracle's two pre-activations (bf16, the rounding points of
+    kernels/pytorch/moe.py:125-139) and the first-order bound on |h_gpu - h| when the GPU's g and u
+    are the same sums accumulated in another order: each may land one bf16 ulp away (plus the
+    fp32-accumulation floor where it is small by cancellation), |silu'| <= 1.1, and silu and the
+    product each round once more."""
+    h_ref = F.silu(g_ref) * u_ref
+    dg = bf16_ulp(g_ref) + floor_g
+    du = bf16_ulp(u_ref) + floor_u
+    s = F.silu(g_ref).float().abs()
+    bound = 1.1 * dg * u_ref.float().abs() + (s + bf16_ulp(s)) * du + bf16_ulp(s) * u_ref.float().abs() \
+        + 2 * bf16_ulp(h_ref) + 1e-30
+    return h_ref, bound
+
+
+def assert_close_rel_abs(got, ref, rtol, atol, what):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    err = (got - ref).abs()
+    bad = ~(err <= atol + rtol * ref.abs())
+    if bad.any():
+        i = int(torch.argmax(err.flatten()))
+        raise AssertionError(f"{what}: {int(bad.sum())} of {bad.numel()} elements out of rtol {rtol} / atol {atol}; "
+                             f"max err {err.flatten()[i].item():.4g} at ref {ref.flatten()[i].item():.4g}")
+
+
+# ------------------------------------------------------------------ GPU chain
+def gpu_chain(x, routing, wg, wu, wd, gates, K, fp8=False, qweights=None, want_plans=False):
+    """x [T, D] bf16 (device); routing: dict of device tensors (offsets, gate_index, reverse_index);
+    wg, wu [E, D, H] and wd [E, H, O] views (device); gates [T, K] bf16.  fp8: qweights =
+    ((qg, sg), (qu, su), (qd, sd)) quantised once beforehand.  Returns the intermediates."""
+    from fast_moe_amd.kernels.hip import ops
+    T = x.shape[0]
+    R = T * K
+    out = {}
+    off, gi, rev = routing["offsets"], routing["gate_index"], routing["reverse_index"]
+    with torch.no_grad():
+        if fp8:
+            (qg, sg), (qu, su), (qd, sd) = qweights
+            qx, sx = ops.quant_rows_fp8(x)
+            kw1 = dict(total_rows=R, row_index=gi, index_div=K, b2=qu, epilogue=2, a_scale=sx, b_scale=sg, b2_scale=su)
+            hidden = ops.grouped_gemm(off, qx, qg, **kw1)
+            qh, sh = ops.quant_rows_fp8(hidden)
+            kw2 = dict(total_rows=R, a_scale=sh, b_scale=sd)
+            rows = ops.grouped_gemm(off, qh, qd, **kw2)
+            out.update(qx=qx, sx=sx, qh=qh, sh=sh)
+            if want_plans:
+                out["plans"] = (ops.grouped_gemm(off, qx, qg, plan_only=True, **kw1),
+                                ops.grouped_gemm(off, qh, qd, plan_only=True, **kw2))
+        else:
+            kw1 = dict(total_rows=R, row_index=gi, index_div=K, b2=wu, epilogue=2)
+            hidden = ops.grouped_gemm(off, x, wg, **kw1)
+            rows = ops.grouped_gemm(off, hidden, wd, total_rows=R)
+            if want_plans:
+                out["plans"] = (ops.grouped_gemm(off, x, wg, plan_only=True, **kw1),
+                                ops.grouped_gemm(off, hidden, wd, total_rows=R, plan_only=True))
+        y = ops.combine(rows, rev, gates, gi)
+    out.update(hidden=hidden, rows=rows, y=y)
+    return out
+
+
+# ------------------------------------------------------------------ oracle pieces on samples
+def mini_offsets(experts, E):
+    """offsets [E+1] of a sample of rows whose expert ids (ascending) are given."""
+    counts = torch.bincount(experts, minlength=E)
+    return torch.cat([torch.zeros(1, dtype=torch.int64), torch.cumsum(counts, 0)])
+
+
+def sample_rows(offsets, R, n, seed):
+    """n distinct routed rows (ascending, hence expert-sorted) with their expert ids."""
+    g = torch.Generator().manual_seed(seed)
+    rows = torch.sort(torch.randperm(R, generator=g)[:n]).values
+    experts = torch.searchsorted(offsets[1:].contiguous(), rows, right=True)
+    return rows, experts
+
+
+def oracle_gemm1_rows(x_rows, experts, E, wg, wu, fp32):
+    """SwiGLU GEMM of the oracle on sampled rows: x_rows [n, D] = the token row of each sampled
+    routed row (expert-sorted), weights [E, D, H] CPU views.  fp32: silu(g) * u accumulated and
+    kept in fp32.  Otherwise the two bf16 pre-activations (g, u) of kernels/pytorch/moe.py:125-139."""
+    n = x_rows.shape[0]
+    off = mini_offsets(experts, E)
+    idx = torch.arange(n).view(-1, 1)
+    if fp32:
+        used = torch.unique(experts).tolist()
+        # only the sampled experts are upcast (an fp32 copy of every expert would be 3x the bf16 tensors)
+        out = torch.empty(n, wg.shape[2], dtype=torch.float32)
+        for e in used:
+            sel = experts == e
+            xe = x_rows[sel].float()
+            out[sel] = F.silu(xe @ wg[e].float()) * (xe @ wu[e].float())
+        return out
+    return (o_moe.index_select_jagged_bmm(off, idx, x_rows, wg, None),
+            o_moe.index_select_jagged_bmm(off, idx, x_rows, wu, None))
+
+
+def oracle_gemm2_rows(h_rows, experts, E, wd, fp32):
+    n = h_rows.shape[0]
+    if fp32:
+        out = torch.empty(n, wd.shape[2], dtype=torch.float32)
+        for e in torch.unique(experts).tolist():
+            sel = experts == e
+            out[sel] = h_rows[sel].float() @ wd[e].float()
+        return out
+    return o_moe.silu_jagged_bmm(mini_offsets(experts, E), h_rows, wd, None, has_silu=False)
+
+
+def abs_sum_gemm(a_rows, experts, w):
+    """sum_k |a[r, k]| * |w[e(r), k, n]|: the scale of the fp32-accumulation error of a row."""
+    out = torch.empty(a_rows.shape[0], w.shape[2], dtype=torch.float32)
+    for e in torch.unique(experts).tolist():
+        sel = experts == e
+        out[sel] = a_rows[sel].float().abs() @ w[e].float().abs()
+    return out
+
+
+def oracle_fp8_rows(q_rows, s_rows, experts, E, qw_codes, s_w):
+    """The oracle's emulated fp8 linear (kernels/pytorch/moe_fp8.py:127-137) on sampled rows:
+    q_rows uint8 codes [n, K], s_rows [n], weight codes [E, N, K] uint8, scales [E, N]."""
+    sizes = torch.bincount(experts, minlength=E).tolist()
+    qa = o_fp8.dequant(q_rows)
+    outs = o_fp8.fp8_linear_per_expert(list(qa.split(sizes)), list(s_rows.split(sizes)), o_fp8.LazyDequant(qw_codes), s_w,
+                                       None, BF16)
+    return torch.cat(outs, dim=0)
+
+
+def abs_sum_fp8(q_rows, s_rows, experts, qw_codes, s_w):
+    out = torch.empty(q_rows.shape[0], qw_codes.shape[1], dtype=torch.float32)
+    qa = o_fp8.dequant(q_rows).abs()
+    for e in torch.unique(experts).tolist():
+        sel = experts == e
+        acc = qa[sel] @ o_fp8.dequant(qw_codes[e]).abs().T
+        out[sel] = acc / (s_rows[sel][:, None] * s_w[e][None, :])
+    return out
+
+
+def subset_problem(topk_subset, E):
+    """Routing tensors (CPU, torch) of a subset of tokens taken as a problem of its own."""
+    meta = o_routing.routing_metadata(np.ascontiguousarray(topk_subset.numpy()), E)
+    return {k: torch.from_numpy(np.ascontiguousarray(v)) for k, v in meta.items() if k != "max_seq_len"}
+
+
+def oracle_chain_tokens(x_s, topk_s, E, K, wg, wu, wd, gates_s, fp8, fp32=False, quantized=None):
+    """The oracle's whole chain on a subset of tokens (each token's output depends on no other
+    token, so the subset's outputs must equal the full run's outputs for those tokens)."""
+    r = subset_problem(topk_s, E)
+    idx2 = r["gate_index"].view(-1, K)
+    if fp8:
+        y, _ = o_fp8.swiglu_moe_fp8(r["offsets"], idx2, x_s, wg, None, wu, None, wd, None, r["token_index"], K,
+                                    gates_s, r["gate_index"], quantized=quantized)
+        return y
+    if fp32:
+        # per-expert upcast of the experts the subset uses
+        tok = r["token_index"]
+        exp = torch.searchsorted(r["offsets"][1:].contiguous(), torch.arange(tok.numel()), right=True)
+        h = oracle_gemm1_rows(x_s[tok], exp, E, wg, wu, fp32=True)
+        rows = oracle_gemm2_rows(h, exp, E, wd, fp32=True)
+        return o_moe.mul_merge_k_add(tok, rows, K, gates_s.float(), r["gate_index"])
+    return o_moe.fused_jagged_bmm_swiglu_combine(r["offsets"], idx2, x_s, wg, None, wu, None, wd, None, K, gates_s,
+                                                 r["gate_index"])
+
+
+def check_sampled(E, K, x, topk, gates, route_fn, w_dev, w_cpu, q_dev, q_cpu, fp8, seed, expect_plans=None,
+                  twins=None, n_rows=256, n_tokens=64):
+    """The full-size check shared by the large configurations.
+
+    x [T, D] bf16, topk [T, K] expert ids, gates [T, K] (CPU); route_fn(topk) -> device routing
+    tensors; w_dev / w_cpu = (wg, wu, wd) [E, K, N] views on the device / the CPU; q_dev / q_cpu the
+    e4m3 forms of the GPU library and of the oracle (fp8 only).
+
+    * routed rows sampled per stage, each stage on the GPU's own inputs of that stage: GEMM1 +
+      SwiGLU within the first-order bound of swiglu_ref_and_bound, the row quantisations bit-exact,
+      GEMM2 within 2 bf16 ulps (+ the fp32-accumulation floor);
+    * the merge of every token, on the GPU's own rows: bit-exact;
+    * sampled tokens end to end: bf16 within 1e-2 abs / rel of the fp32-accumulated oracle, e4m3
+      within 3e-2 of the oracle's own fp8 chain;
+    * over the whole batch: a permutation of the tokens permutes the outputs bit for bit, and
+      twin tokens (same row, same experts) give identical outputs."""
+    T = x.shape[0]
+    meta = subset_problem(topk, E)
+    r = route_fn(topk)
+    for key in ("offsets", "gate_index", "reverse_index"):
+        assert torch.equal(r[key].cpu().view(-1), meta[key].view(-1)), key
+    xd = x.cuda()
+    got = gpu_chain(xd, r, *w_dev, gates.cuda(), K, fp8=fp8, qweights=q_dev, want_plans=True)
+    if expect_plans is not None:
+        assert got["plans"] == tuple(expect_plans), got["plans"]
+    y = got["y"].cpu()
+    assert bool(torch.isfinite(y.float()).all())
+    if twins is not None:
+        assert torch.equal(y[twins[0]], y[twins[1]])
+    wg, wu, wd = w_cpu
+    R = T * K
+    rows, experts = sample_rows(meta["offsets"], R, n_rows, seed=seed + 1)
+    tok = meta["token_index"][rows]
+    hidden_s, rows_s = got["hidden"][rows.cuda()].cpu(), got["rows"][rows.cuda()].cpu()
+    if not fp8:
+        g_ref, u_ref = oracle_gemm1_rows(x[tok], experts, E, wg, wu, fp32=False)
+        h_ref, bound = swiglu_ref_and_bound(g_ref, u_ref, BF16_FLOOR * abs_sum_gemm(x[tok], experts, wg),
+                                            BF16_FLOOR * abs_sum_gemm(x[tok], experts, wu))
+        assert_within(hidden_s, h_ref, bound, "GEMM1 + SwiGLU")
+        r_ref = oracle_gemm2_rows(hidden_s, experts, E, wd, fp32=False)
+        assert_ulp_close(rows_s, r_ref, 2, BF16_FLOOR * abs_sum_gemm(hidden_s, experts, wd), "GEMM2")
+    else:
+        (lg, sg), (lu, su), (ld, sd) = q_cpu
+        qx_ref, sx_ref = o_fp8.rowwise_quant_fp8(x)
+        assert torch.equal(got["sx"].cpu(), sx_ref)
+        assert torch.equal(got["qx"].view(torch.uint8).cpu(), qx_ref)
+        g_ref = oracle_fp8_rows(qx_ref[tok], sx_ref[tok], experts, E, lg.codes, sg)
+        u_ref = oracle_fp8_rows(qx_ref[tok], sx_ref[tok], experts, E, lu.codes, su)
+        h_ref, bound = swiglu_ref_and_bound(
+            g_ref, u_ref, FP8_FLOOR * abs_sum_fp8(qx_ref[tok], sx_ref[tok], experts, lg.codes, sg),
+            FP8_FLOOR * abs_sum_fp8(qx_ref[tok], sx_ref[tok], experts, lu.codes, su))
+        assert_within(hidden_s, h_ref, bound, "fp8 GEMM1 + SwiGLU")
+        qh_ref, sh_ref = o_fp8.rowwise_quant_fp8(hidden_s)
+        assert torch.equal(got["sh"][rows.cuda()].cpu(), sh_ref)
+        assert torch.equal(got["qh"].view(torch.uint8)[rows.cuda()].cpu(), qh_ref)
+        r_ref = oracle_fp8_rows(qh_ref, sh_ref, experts, E, ld.codes, sd)
+        assert_ulp_close(rows_s, r_ref, 2, FP8_FLOOR * abs_sum_fp8(qh_ref, sh_ref, experts, ld.codes, sd), "fp8 GEMM2")
+    y_ref = o_moe.mul_merge_k_add(meta["token_index"], got["rows"].cpu(), K, gates, meta["gate_index"])
+    assert torch.equal(y, y_ref), "merge"
+    g = torch.Generator().manual_seed(seed + 2)
+    toks = torch.sort(torch.randperm(T, generator=g)[:n_tokens]).values
+    if fp8:
+        toks[0] = 0                          # row 0 is an outlier row in the fp8 configurations
+        y8 = oracle_chain_tokens(x[toks], topk[toks], E, K, wg, wu, wd, gates[toks], fp8=True, quantized=q_cpu)
+        assert_close_rel_abs(y[toks], y8, 3e-2, 3e-2 * y8.float().abs().max().item(), "fp8 forward")
+    else:
+        y32 = oracle_chain_tokens(x[toks], topk[toks], E, K, wg, wu, wd, gates[toks], fp8=False, fp32=True)
+        assert_close_rel_abs(y[toks], y32, 1e-2, 1e-2, "bf16 forward vs fp32 oracle")
+    perm = torch.randperm(T, generator=g)
+    r2 = route_fn(topk[perm])
+    got2 = gpu_chain(xd[perm.cuda()], r2, *w_dev, gates[perm].cuda(), K, fp8=fp8, qweights=q_dev)
+    assert torch.equal(got2["y"].cpu(), y[perm]), "token permutation"
+    return got

@@ -59,3 +59,20 @@ def assert_bf16_close(got, ref_fp32, rtol=1e-2, atol=1e-2, what=""):
     bad = err > bound
     assert not bad.any(), (f"{what}: {int(bad.sum())} of {bad.numel()} elements out of tolerance; "
                            f"max err {err.max().item():.4g} at ref {ref.flatten()[err.argmax()].item():.4g}")
+
+
+def special_scores(T=64, E=16, seed=3):
+    """Rows with NaN, +-inf, +-0 and all-equal values among ordinary ones (distinct otherwise)."""
+    g = torch.Generator().manual_seed(seed)
+    s = torch.rand(T, E, generator=g)
+    s[1] = float("nan")                       # the usual divergence case: a row of NaN
+    s[2, 3] = float("nan")
+    s[2, 9] = float("nan")
+    s[3, 5] = float("inf")
+    s[4, 7] = float("-inf")
+    s[5] = 0.25                               # all equal
+    s[6, :4] = 0.0
+    s[6, 4:8] = -0.0
+    s[7, 2] = float("nan")
+    s[7, 11] = float("inf")
+    return s

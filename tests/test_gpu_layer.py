@@ -28,7 +28,8 @@ def build_layer(D, H, O, E, seed=0):
 
 
 @pytest.mark.parametrize("B,S,D,H,O,E,k", [(4, 8, 16, 32, 16, 4, 1), (8, 16, 32, 16, 32, 8, 2),
-                                           (2, 512, 256, 512, 256, 8, 2), (4, 512, 1024, 4096, 1024, 8, 2)])
+                                           (2, 512, 256, 512, 256, 8, 2), (4, 512, 1024, 4096, 1024, 8, 2),
+                                           (8, 1024, 1024, 4096, 1024, 8, 2)])    # the last: 8192 tokens
 def test_layer_matches_oracle(B, S, D, H, O, E, k):
     """Shapes of modules/tests/test_kernel_parity.py:29-90 plus the plumbing configuration."""
     print(f"layer B={B} S={S} D={D} H={H} O={O} E={E} k={k}", flush=True)

@@ -160,22 +160,45 @@ def test_silu_quant_and_weight_quant():
     assert np.array_equal(s3.cpu().numpy(), s3_ref)
 
 
-def test_fp8_operator_reuses_cached_weight_quantisation():
-    """index_select_jagged_bmm(fp8=True) quantises a weight once and again only after an update."""
+def test_fp8_operators_requantise_every_call_and_take_a_kept_pair():
+    """The fp8 operators quantise their weight on every call, as the reference does
+    (kernels/pytorch/moe_fp8.py:111): updates the version counter cannot see -- writes through
+    ``.data``, an optimizer step -- are picked up.  The kept pair is opt-in (``fp8_weight=``)."""
     from fast_moe_amd.kernels import moe_fp8
     from helpers import make_routing, randn
     r = make_routing(512, 8, 2, seed=5)
     x = randn((512, 128), 1).cuda()
-    w = (randn((8, 128, 96), 2) * 128 ** -0.5).cuda()
+    w = torch.nn.Parameter((randn((8, 128, 96), 2) * 128 ** -0.5).cuda())
     off, idx = r["offsets"].cuda(), r["index"].cuda()
     cache = moe_fp8.weight_quant_cache
     cache.clear()
     h0, m0 = cache.hits, cache.misses
     with torch.no_grad():
         y1 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
+        w.data.mul_(2.0)                                  # invisible to w._version
         y2 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
-        assert (cache.hits - h0, cache.misses - m0) == (1, 1) and torch.equal(y1, y2)
-        w.mul_(2.0)
-        y3 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
-    assert cache.misses - m0 == 2
-    torch.testing.assert_close(y3.float(), 2 * y1.float(), rtol=0, atol=0)   # a power of two: exact
+        torch.testing.assert_close(y2.float(), 2 * y1.float(), rtol=0, atol=0)   # a power of two: exact
+        assert (cache.hits - h0, cache.misses - m0) == (0, 0)                    # the operator does not cache
+        # the kept pair: same bits as the default path, until the weight moves
+        pair = moe_fp8.cached_quantize_expert_weights(w)
+        assert moe_fp8.cached_quantize_expert_weights(w)[0] is pair[0]
+        y3 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True, fp8_weight=pair)
+        assert torch.equal(y3, y2)
+    opt = torch.optim.SGD([w], lr=0.5)
+    w.grad = torch.ones_like(w) * 0.01
+    opt.step()                                            # an in-place update: the version counter moves
+    with torch.no_grad():
+        pair2 = moe_fp8.cached_quantize_expert_weights(w)
+        assert pair2[0] is not pair[0]
+        y4 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True)
+        y5 = moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True, fp8_weight=pair2)
+        assert torch.equal(y4, y5) and not torch.equal(y4, y2)
+        fresh = moe_fp8.quantize_expert_weights(w)
+        assert torch.equal(fresh[0].view(torch.uint8), pair2[0].view(torch.uint8)) and torch.equal(fresh[1], pair2[1])
+        # a write through .data leaves the cache stale until it is invalidated
+        w.data.mul_(2.0)
+        assert moe_fp8.cached_quantize_expert_weights(w)[0] is pair2[0]
+        cache.invalidate(w)
+        assert torch.equal(moe_fp8.cached_quantize_expert_weights(w)[1], pair2[1] * 0.5)
+    with pytest.raises(ValueError):
+        moe_fp8.index_select_jagged_bmm(0, off, idx, x, w, None, fp8=True, fp8_weight=(pair[0][:4], pair[1]))

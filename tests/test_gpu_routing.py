@@ -49,6 +49,29 @@ def test_route_topk_ties_and_no_renorm():
     assert got["topk_idx"].cpu().tolist() == [[0, 1, 2, 3]] * 37
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("E", [16, 64, 128])
+def test_route_topk_nan_inf_and_equal_rows(E, dtype):
+    """Scores after a divergence (rows of NaN, single NaN, +-inf, +-0, all-equal rows): NaN ranks
+    above +inf as in torch.topk, every token still fills K distinct slots with ids in [0, E), the
+    integer outputs equal the oracle's, lengths sum to T*K, and the gates carry the same NaN."""
+    from fast_moe_amd.kernels.hip import ops
+    from tests.helpers import special_scores
+    scores = special_scores(T=64, E=E, seed=E).to(dtype)
+    name = "bf16" if dtype == torch.bfloat16 else "fp32"
+    for K in (1, 4, 8):
+        for renorm in (True, False):
+            ref = o_routing.route(scores.float().numpy(), K, dtype=name, renorm=renorm)
+            got = ops.route_topk(scores.cuda(), K, renorm=renorm)
+            idx = got["topk_idx"].cpu()
+            assert int(idx.min()) >= 0 and int(idx.max()) < E
+            assert all(len(set(row)) == K for row in idx.tolist())
+            assert int(got["lengths"].sum()) == 64 * K
+            for key in INT_KEYS:
+                assert np.array_equal(got[key].cpu().numpy().reshape(ref[key].shape), ref[key]), (key, K, renorm)
+            assert np.array_equal(got["gates"].float().cpu().numpy(), ref["gates"], equal_nan=True), (K, renorm)
+
+
 @pytest.mark.parametrize("T,E,K,dtype", [(16384, 64, 8, torch.float32), (8192, 8, 2, torch.bfloat16),
                                          (32768, 128, 8, torch.float32)])
 def test_route_topk_full_size(T, E, K, dtype):

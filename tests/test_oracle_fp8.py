@@ -151,3 +151,27 @@ def test_silu_quant_against_torch_ops():
     assert np.array_equal(s, s_ref.numpy())
     # exp() of two libraries may differ in the last fp32 bit before the bf16 rounding
     assert np.mean(q != q_ref) < 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_library_cast_path_equals_bit_level_path(dtype):
+    """oracle.moe_fp8.rowwise_quant_fp8 has two casts: the bit-level encoder and, for operands of
+    10^9 elements, Tensor.to(float8_e4m3fn).  Same codes and scales on random rows, outlier rows,
+    zero rows, rows whose scaled values land in the subnormal range, and inf / NaN rows."""
+    from oracle import moe_fp8 as o8
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(3, 40, 256, generator=g)
+    a[0, ::7] *= 100
+    a[1, 3] = 0
+    a[1, 4, 1:] *= 2.0 ** -12            # one large entry, the rest rounds into subnormals / zero
+    a[2, 5, 9] = float("inf")
+    a[2, 6, 11] = float("nan")
+    a = a.to(dtype)
+    qb, sb = o8.rowwise_quant_fp8(a, cast="bits")
+    qt, st = o8.rowwise_quant_fp8(a, cast="torch")
+    assert torch.equal(sb, st)
+    assert torch.equal(qb, qt)
+    big = torch.randn(1 << 11, 1 << 11, generator=g).to(dtype)      # above the size switch
+    q_auto, s_auto = o8.rowwise_quant_fp8(big)
+    q_bits, s_bits = o8.rowwise_quant_fp8(big[:64], cast="bits")
+    assert torch.equal(q_auto[:64], q_bits) and torch.equal(s_auto[:64], s_bits)

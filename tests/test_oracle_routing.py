@@ -5,6 +5,7 @@ import torch
 from torch.nn import functional as F
 
 from oracle import routing
+from tests.helpers import special_scores
 
 
 def brute_force_routing(topk, E):
@@ -118,3 +119,35 @@ def test_round_to_bf16_matches_torch():
     x = torch.randn(100000, generator=g) * torch.exp(torch.randn(100000, generator=g) * 10)
     ref = x.to(torch.bfloat16).float().numpy()
     assert np.array_equal(routing.round_to_bf16(x.numpy()), ref)
+
+
+def test_top_k_total_order_with_nan_inf_and_ties():
+    """torch.topk ranks NaN above +inf; ties go to the lower expert id (canonical).  Every row
+    yields k distinct ids in range whatever it holds."""
+    s = special_scores()
+    T, E = s.shape
+    for k in (1, 2, 5, 16):
+        idx, _ = routing.select_top_k(s.numpy(), k, renorm=False)
+        assert idx.min() >= 0 and idx.max() < E
+        assert all(len(set(row)) == k for row in idx.tolist())
+        ref = s.topk(k, dim=1).indices
+        for t in range(T):
+            if t in (1, 5, 6):          # ties at the cut: the canonical rule decides, checked below
+                continue
+            if t == 2 and k == 1:       # two NaN tie for one slot
+                continue
+            assert set(idx[t].tolist()) == set(ref[t].tolist()), (t, k)
+    idx, _ = routing.select_top_k(s.numpy(), 5, renorm=False)
+    assert idx[1].tolist() == [0, 1, 2, 3, 4] and idx[5].tolist() == [0, 1, 2, 3, 4]
+    assert idx[2].tolist()[:2] == [3, 9]                    # the NaN first, in id order
+    assert idx[7].tolist()[:2] == [2, 11]                   # NaN above +inf
+    assert idx[3].tolist()[0] == 5
+    assert 7 not in routing.select_top_k(s.numpy(), E - 1, renorm=False)[0][4].tolist()   # -inf last
+    key = routing.order_key(np.array([-0.0, 0.0, -1.0, 1.0, np.inf, -np.inf, np.nan, -np.nan], dtype=np.float32))
+    assert key[0] == key[1] and key[6] == key[7] and key[5] < key[2] < key[0] < key[3] < key[4] < key[6]
+    # gates of a row with a NaN among the selected: F.normalize propagates NaN to the whole row
+    _, gates = routing.select_top_k(s.numpy(), 4)
+    ref = F.normalize(torch.gather(s, 1, torch.from_numpy(routing.select_top_k(s.numpy(), 4)[0])), p=1, dim=1)
+    assert np.array_equal(np.isnan(gates), torch.isnan(ref).numpy())
+    ok = ~np.isnan(gates)
+    assert np.allclose(gates[ok], ref.numpy()[ok], rtol=1e-6, atol=0)
