@@ -14,6 +14,8 @@
 //                      its expert segment
 #include "common.h"
 
+#include <mutex>
+
 namespace fmoe {
 namespace {
 
@@ -391,23 +393,21 @@ extern "C" size_t fmoe_route_workspace_bytes(int64_t T, int E, int K) {
     return make_plan(T, E, K).total_bytes;
 }
 
-extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
-                               int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
-                               int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
-                               void* workspace, size_t workspace_bytes, fmoe_stream_t stream_) {
-    hipStream_t stream = (hipStream_t)stream_;
-    if (int rc = check_common(T, E, K, workspace, workspace_bytes, "fmoe_route_topk")) return rc;
-    FMOE_REQUIRE(K <= E, "fmoe_route_topk: K=%d > E=%d", K, E);
-    FMOE_REQUIRE(renorm >= 0 && renorm <= 3, "fmoe_route_topk: gate mode %d is not one of 0..3", renorm);
-    FMOE_REQUIRE(score_dtype == FMOE_F32 || score_dtype == FMOE_BF16,
-                 "fmoe_route_topk: scores must be fp32 or bf16");
-    FMOE_REQUIRE(lengths && offsets, "fmoe_route_topk: lengths/offsets are NULL");
+static int route_topk_impl(const char* who, const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
+                           int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
+                           int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
+                           void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    if (int rc = check_common(T, E, K, workspace, workspace_bytes, who)) return rc;
+    FMOE_REQUIRE(K <= E, "%s: K=%d > E=%d", who, K, E);
+    FMOE_REQUIRE(renorm >= 0 && renorm <= 3, "%s: gate mode %d is not one of 0..3", who, renorm);
+    FMOE_REQUIRE(score_dtype == FMOE_F32 || score_dtype == FMOE_BF16, "%s: scores must be fp32 or bf16", who);
+    FMOE_REQUIRE(lengths && offsets, "%s: lengths/offsets are NULL", who);
     if (T == 0) {
         empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets);
-        return check_launch("fmoe_route_topk");
+        return check_launch(who);
     }
     FMOE_REQUIRE(scores && topk_idx && gates && gate_index && token_index && reverse_index,
-                 "fmoe_route_topk: NULL tensor pointer");
+                 "%s: NULL tensor pointer", who);
     const RoutePlan plan = make_plan(T, E, K);
     uint16_t* compact = (uint16_t*)workspace;
     int32_t* chunk_hist = (int32_t*)((char*)workspace + plan.compact_bytes);
@@ -417,6 +417,69 @@ extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, i
     if (rc) return rc;
     return launch_sort(compact, chunk_hist, plan, T, E, K, lengths, offsets, gate_index, token_index,
                        reverse_index, stream);
+}
+
+extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
+                               int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
+                               int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
+                               void* workspace, size_t workspace_bytes, fmoe_stream_t stream_) {
+    return route_topk_impl("fmoe_route_topk", scores, score_dtype, T, E, K, renorm, topk_idx, gates, lengths,
+                           offsets, gate_index, token_index, reverse_index, workspace, workspace_bytes,
+                           (hipStream_t)stream_);
+}
+
+// ------------------------------------------------------------ allocation-free variant
+// The routing scratch (one uint16 expert id per routed position + the per-chunk histograms) in
+// device memory that belongs to the library image: one copy per GPU the library runs on, held
+// until the process ends.  In host code `scratch` is only a handle for hipGetSymbolAddress;
+// the address kernels and copies use is the per-device pointer looked up below.
+static constexpr size_t kStaticCompactBytes = (size_t)FMOE_ROUTE_STATIC_MAX_POSITIONS * sizeof(uint16_t);
+static constexpr size_t kStaticHistBytes = (size_t)kMaxChunks * FMOE_ROUTE_STATIC_MAX_EXPERTS * sizeof(int32_t);
+static constexpr size_t kStaticScratchBytes = kStaticCompactBytes + kStaticHistBytes + 512;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];     // device address of `scratch` on each GPU, 0 = not looked up yet
+static std::mutex g_scratch_mutex;
+
+// Device address of this GPU's copy of `scratch` (looked up once per device, with that device current).
+static int static_scratch(void** out, const char* who) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(FMOE_ERR_LAUNCH, "%s: no current device (or device index beyond %d)", who, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        const hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || ptr == nullptr)
+            return fail(FMOE_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev,
+                        hipGetErrorString(err));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return FMOE_OK;
+}
+
+extern "C" int fmoe_route_topk_static(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
+                                      int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
+                                      int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
+                                      fmoe_stream_t stream_) {
+    const char* who = "fmoe_route_topk_static";
+    FMOE_REQUIRE(T >= 0 && E >= 1 && K >= 1, "%s: need T >= 0, E >= 1, K >= 1 (T=%lld E=%d K=%d)", who,
+                 (long long)T, E, K);
+    FMOE_REQUIRE(E <= FMOE_ROUTE_STATIC_MAX_EXPERTS, "%s: E=%d exceeds the %d experts the built-in scratch holds",
+                 who, E, FMOE_ROUTE_STATIC_MAX_EXPERTS);
+    FMOE_REQUIRE(T <= FMOE_ROUTE_STATIC_MAX_POSITIONS && T * (int64_t)K <= FMOE_ROUTE_STATIC_MAX_POSITIONS,
+                 "%s: T*K=%lld routed positions exceed the %d the built-in scratch holds (use fmoe_route_topk "
+                 "with a workspace)", who, (long long)T * K, FMOE_ROUTE_STATIC_MAX_POSITIONS);
+    if (make_plan(T, E, K).total_bytes > kStaticScratchBytes)
+        return fail(FMOE_ERR_WORKSPACE, "%s: the call needs %zu B of scratch, the built-in buffer has %zu B", who,
+                    make_plan(T, E, K).total_bytes, kStaticScratchBytes);
+    void* ptr = nullptr;
+    if (int rc = static_scratch(&ptr, who)) return rc;
+    // nothing in the buffer has to start at zero: the first two kernels overwrite every byte the later ones read
+    return route_topk_impl(who, scores, score_dtype, T, E, K, renorm, topk_idx, gates, lengths, offsets, gate_index,
+                           token_index, reverse_index, ptr, kStaticScratchBytes, (hipStream_t)stream_);
 }
 
 extern "C" int fmoe_route_from_topk(const int64_t* topk_idx, int64_t T, int E, int K, int64_t* lengths,

@@ -22,8 +22,9 @@ EXPORTED_SYMBOLS = (
     "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_grouped_gemm_plan",
     "fmoe_combine",
     "fmoe_silu_mul", "fmoe_transpose_last2", "fmoe_jagged_transpose", "fmoe_segment_colsum",
-    "fmoe_swiglu_bwd", "fmoe_combine_bwd", "fmoe_gather_rows",
+    "fmoe_swiglu_bwd", "fmoe_combine_bwd", "fmoe_gather_rows", "fmoe_route_topk_static",
 )
+ROUTE_STATIC_MAX_POSITIONS, ROUTE_STATIC_MAX_EXPERTS = 1 << 20, 512
 
 
 class GemmDesc(ctypes.Structure):
@@ -72,6 +73,8 @@ def load() -> ctypes.CDLL:
     lib.fmoe_route_topk.restype = c_int
     lib.fmoe_route_topk.argtypes = [c_void_p, c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 7 + [
         c_void_p, c_size_t, c_void_p]
+    lib.fmoe_route_topk_static.restype = c_int
+    lib.fmoe_route_topk_static.argtypes = [c_void_p, c_int, c_int64, c_int, c_int, c_int] + [c_void_p] * 7 + [c_void_p]
     lib.fmoe_route_from_topk.restype = c_int
     lib.fmoe_route_from_topk.argtypes = [c_void_p, c_int64, c_int, c_int] + [c_void_p] * 6 + [
         c_void_p, c_size_t, c_void_p]

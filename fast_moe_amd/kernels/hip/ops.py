@@ -60,9 +60,13 @@ def _rows_contiguous(t: torch.Tensor) -> torch.Tensor:
 GATE_RAW, GATE_L1, GATE_SOFTMAX_ALL, GATE_SOFTMAX_TOPK = 0, 1, 2, 3
 
 
-def route_topk(scores: torch.Tensor, k: int, renorm=True) -> Dict[str, torch.Tensor]:
+def route_topk(scores: torch.Tensor, k: int, renorm=True, static_scratch: bool = False,
+               out: Optional[Dict[str, torch.Tensor]] = None) -> Dict[str, torch.Tensor]:
     """scores [T, E] (fp32 / bf16 gate probabilities, or router logits for the softmax modes)
-    -> routing tensors, see fmoe_route_topk.  ``renorm``: bool, or one of the GATE_* modes."""
+    -> routing tensors, see fmoe_route_topk.  ``renorm``: bool, or one of the GATE_* modes.
+    ``static_scratch``: fmoe_route_topk_static, whose scratch is built into the library (no
+    workspace allocation; T*k <= 2^20, E <= 512).  ``out``: a dict of a previous call with the
+    same shapes, written in place (with static_scratch the call then allocates nothing)."""
     dev = _need_cuda("route_topk", scores)
     if scores.ndim != 2:
         raise ValueError("route_topk: scores must be [T, E]")
@@ -71,16 +75,28 @@ def route_topk(scores: torch.Tensor, k: int, renorm=True) -> Dict[str, torch.Ten
     scores = scores.contiguous()
     T, E = scores.shape
     i64 = dict(dtype=torch.int64, device=dev)
-    out = {
-        "topk_idx": torch.empty((T, k), **i64),
-        "gates": torch.empty((T, k), dtype=scores.dtype, device=dev),
-        "lengths": torch.empty((E,), **i64),
-        "offsets": torch.empty((E + 1,), **i64),
-        "gate_index": torch.empty((T * k,), **i64),
-        "token_index": torch.empty((T * k,), **i64),
-        "reverse_index": torch.empty((T, k), **i64),
-    }
+    if out is None:
+        out = {
+            "topk_idx": torch.empty((T, k), **i64),
+            "gates": torch.empty((T, k), dtype=scores.dtype, device=dev),
+            "lengths": torch.empty((E,), **i64),
+            "offsets": torch.empty((E + 1,), **i64),
+            "gate_index": torch.empty((T * k,), **i64),
+            "token_index": torch.empty((T * k,), **i64),
+            "reverse_index": torch.empty((T, k), **i64),
+        }
+    elif (tuple(out["topk_idx"].shape) != (T, k) or out["gates"].dtype != scores.dtype
+          or out["lengths"].numel() != E or out["gate_index"].device != dev):
+        raise ValueError("route_topk: `out` was made for other shapes")
     lib = _lib.load()
+    if static_scratch:
+        rc = lib.fmoe_route_topk_static(
+            scores.data_ptr(), _DTYPE_CODE[scores.dtype], T, E, k, int(renorm),
+            out["topk_idx"].data_ptr(), out["gates"].data_ptr(), out["lengths"].data_ptr(),
+            out["offsets"].data_ptr(), out["gate_index"].data_ptr(), out["token_index"].data_ptr(),
+            out["reverse_index"].data_ptr(), _stream(scores))
+        _lib.check(rc, "fmoe_route_topk_static")
+        return out
     ws_bytes = lib.fmoe_route_workspace_bytes(T, E, k)
     ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
     rc = lib.fmoe_route_topk(

@@ -93,6 +93,26 @@ int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K
                     void* workspace, size_t workspace_bytes, fmoe_stream_t stream);
 
 /*
+ * fmoe_route_topk without a workspace argument and without any allocation: the scratch lives in
+ * device memory that is part of the library image (3 MiB per GPU the library runs on, held until
+ * the process ends).  No counterpart in the reference.  For callers that cannot allocate: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments
+ * and results as fmoe_route_topk, bit for bit.
+ * Limits: T * K <= FMOE_ROUTE_STATIC_MAX_POSITIONS, E <= FMOE_ROUTE_STATIC_MAX_EXPERTS; larger
+ * calls are turned away with FMOE_ERR_ARGUMENT (use fmoe_route_topk with a workspace).
+ * Every call on a GPU uses that GPU's one buffer: calls that may overlap on one GPU (two
+ * streams, two threads) race; calls on one stream, or ordered by events, do not.  The first call
+ * on a device looks the buffer's address up (hipGetSymbolAddress); make that call outside a
+ * graph capture.
+ */
+#define FMOE_ROUTE_STATIC_MAX_POSITIONS (1 << 20)
+#define FMOE_ROUTE_STATIC_MAX_EXPERTS 512
+int fmoe_route_topk_static(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
+                           int64_t* topk_idx, void* gates, int64_t* lengths, int64_t* offsets,
+                           int64_t* gate_index, int64_t* token_index, int64_t* reverse_index,
+                           fmoe_stream_t stream);
+
+/*
  * The same routing tensors for a caller that already holds the selected expert
  * ids (the generator of kernels/tests/moe_test.py:191-197,241: topk -> stable
  * sort -> scatter_add -> complete cumsum).  topk_idx values must lie in [0, E);

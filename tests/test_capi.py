@@ -34,6 +34,16 @@ def test_every_declared_symbol_is_exported(lib):
     assert sorted(_lib.EXPORTED_SYMBOLS) == names
 
 
+def test_static_routing_rejects_oversize_calls_without_a_gpu(lib):
+    """fmoe_route_topk_static checks its limits before it touches a device."""
+    bad = ctypes.c_void_p(16)
+    args = [bad] * 7 + [None]
+    assert lib.fmoe_route_topk_static(bad, 0, (1 << 20) // 8 + 1, 8, 8, 1, *args) == 1
+    assert b"routed positions exceed" in lib.fmoe_last_error()
+    assert lib.fmoe_route_topk_static(bad, 0, 4, 513, 2, 1, *args) == 1
+    assert b"experts" in lib.fmoe_last_error()
+
+
 def test_gemm_desc_layout_matches_header():
     from fast_moe_amd.kernels.hip._lib import GemmDesc
     text = open(HEADER).read()
