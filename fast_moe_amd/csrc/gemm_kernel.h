@@ -948,7 +948,7 @@ __device__ __forceinline__ int lds_off64(int row, int chunk) {   // 64-byte rows
 // hand below).
 __device__ __forceinline__ void dma16(const uint8_t* base, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n"
-                 :: "v"(voff), "s"(base), "s"(lds_addr) : "memory");
+                 :: "v"(voff), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
 __device__ __forceinline__ int uniform_lane(int v, int src_lane) {

@@ -275,6 +275,13 @@ __global__ __launch_bounds__(kWave) void scatter_kernel(const uint16_t* __restri
             run += wave_bcast(inc, kWave - 1);
         }
         if (c == 0 && lane == 0) offsets[E] = run;
+        // positions dropped for an out-of-range expert id leave a tail behind the last expert's
+        // rows: it holds zeros rather than whatever the buffer held (normally the tail is empty)
+        if (c == 0)
+            for (long long i = run + lane; i < (long long)num_tokens * K; i += kWave) {
+                gate_index[i] = 0;
+                token_index[i] = 0;
+            }
     }
     __syncthreads();
     const int tpi = kWave / K;
@@ -314,6 +321,8 @@ __global__ __launch_bounds__(kWave) void scatter_kernel(const uint16_t* __restri
             gate_index[dst] = p;
             token_index[dst] = t;
             reverse_index[t * K + rank] = dst;
+        } else if (live) {
+            reverse_index[t * K + rank] = 0;    // a dropped position (out-of-range id): sorts last in its token
         }
     }
 }

@@ -5,6 +5,7 @@ memory and streams only; every computation below happens in libfastmoe_hip.so.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -109,7 +110,9 @@ def route_topk(scores: torch.Tensor, k: int, renorm=True, static_scratch: bool =
 
 
 def route_from_topk(topk_idx: torch.Tensor, num_experts: int) -> Dict[str, torch.Tensor]:
-    """topk_idx [T, K] int64 expert ids -> routing tensors, see fmoe_route_from_topk."""
+    """topk_idx [T, K] int64 expert ids -> routing tensors, see fmoe_route_from_topk.  Ids outside
+    [0, num_experts) are dropped and counted in ``bad_count`` (a device tensor: reading it
+    synchronises); with FMOE_CHECK_ROUTING=1 in the environment the call checks it and raises."""
     dev = _need_cuda("route_from_topk", topk_idx)
     if topk_idx.ndim != 2:
         raise ValueError("route_from_topk: topk_idx must be [T, K]")
@@ -133,6 +136,10 @@ def route_from_topk(topk_idx: torch.Tensor, num_experts: int) -> Dict[str, torch
         out["gate_index"].data_ptr(), out["token_index"].data_ptr(), out["reverse_index"].data_ptr(),
         out["bad_count"].data_ptr(), ws.data_ptr(), ws_bytes, _stream(topk_idx))
     _lib.check(rc, "fmoe_route_from_topk")
+    if os.environ.get("FMOE_CHECK_ROUTING") == "1":     # debugging aid: costs a host synchronisation
+        bad = int(out["bad_count"])
+        if bad:
+            raise ValueError(f"route_from_topk: {bad} expert ids outside [0, {E})")
     return out
 
 

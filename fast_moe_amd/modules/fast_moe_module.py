@@ -20,14 +20,7 @@ from torch.autograd.profiler import record_function
 from ..kernels.hip import ops
 from ..kernels.hip._lib import EPI_NONE, EPI_SILU
 from ..kernels.utils import KernelType, require_hip_kernel
-
-
-def _create_fused_mlp_weights(num_mlps: int, in_dim: int, out_dim: int) -> torch.Tensor:
-    """utils/utils.py:38-42: one xavier-uniform [in_dim, out_dim] matrix per expert."""
-    t = torch.empty(size=(num_mlps, in_dim, out_dim))
-    for i in range(num_mlps):
-        torch.nn.init.xavier_uniform_(t[i])
-    return t
+from ..utils.utils import _create_fused_mlp_weights
 
 
 class GatingNetwork(nn.Module):

@@ -117,7 +117,9 @@ int fmoe_route_topk_static(const void* scores, int score_dtype, int64_t T, int E
  * ids (the generator of kernels/tests/moe_test.py:191-197,241: topk -> stable
  * sort -> scatter_add -> complete cumsum).  topk_idx values must lie in [0, E);
  * out-of-range ids are counted into no expert and reported through
- * `bad_count` (device int64, may be NULL).  Limits: E <= 1024, K <= 64.
+ * `bad_count` (device int64, may be NULL); the positions they leave unfilled (the
+ * tail of gate_index / token_index behind offsets[E], the last slots of their
+ * token's reverse_index row) hold 0.  Limits: E <= 1024, K <= 64.
  */
 int fmoe_route_from_topk(const int64_t* topk_idx, int64_t T, int E, int K,
                          int64_t* lengths, int64_t* offsets, int64_t* gate_index,

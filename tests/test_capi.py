@@ -224,3 +224,17 @@ def test_reference_helper_names_import_without_a_gpu():
     cfg = SGConfig(model_d=8, num_experts=4, num_activated_experts=2)
     assert cfg.loss_coef == 1e-2 and not cfg.enable_noisy_gating
     assert MRNOutput._fields == ("x", "loss", "load")
+
+
+def test_reference_import_paths_resolve():
+    """The import statements of code written against the reference's operator path."""
+    from fast_moe import FastMoELayer, KernelType
+    from fast_moe.kernels import moe as m1
+    from fast_moe.kernels.moe import index_select_jagged_bmm, mul_merge_k_add, silu_jagged_bmm_combine
+    from fast_moe.kernels.moe_fp8 import index_select_jagged_bmm as bmm_fp8
+    from fast_moe.kernels.utils import KernelType as K2
+    from fast_moe.modules.fast_moe_module import FastMoELayer as L2
+    from fast_moe.utils.utils import _compute_top_logits, _dispatch
+    import fast_moe_amd.kernels.moe as real
+    assert m1 is real and index_select_jagged_bmm is real.index_select_jagged_bmm
+    assert K2 is KernelType and L2 is FastMoELayer and callable(bmm_fp8) and callable(_dispatch)
