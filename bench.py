@@ -2,7 +2,7 @@
 """Benchmark of the MoE-forward hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_bf16|c4_fp8|c2_bf16|c5_bf16|c5_fp8]
-                    [--tokens T] [--no-cpu-baseline] [--no-extra]
+                    [--tokens T] [--no-cpu-baseline] [--no-extra] [--sample-clock] [--dense-reference]
 
 A step is one forward pass of the hot path over one batch of synthetic input that is
 already resident in HBM: top-k routing from the gate probabilities, the gather +
@@ -10,6 +10,13 @@ grouped GEMM with its SiLU / SwiGLU epilogue, (fp8: the row-wise quantisations),
 the down-projection GEMM and the weighted merge.  The gate Linear + softmax that
 produce the probabilities stay torch calls and are outside the step, as they are
 outside the FLOP count.  Prints ONE JSON line.
+
+Timing: `value` / `ms_per_step` come from exactly K back-to-back steps between two device
+synchronisations (hot caches, the steady state of a serving loop).  Beside it: per-step HIP-event
+samples (median, p95), the same with a 512 MiB buffer rewritten before every step so that neither
+L2 nor the 256 MB last-level cache holds anything of the previous step (`cold`), and per-kernel
+durations from HIP events over max(K, 100) launches after 25 warm-up launches (the reference's
+do_bench(warmup=25, rep=100), kernels/benchmarks/timer.py:174-198).
 """
 from __future__ import annotations
 
@@ -17,7 +24,10 @@ import argparse
 import json
 import math
 import os
+import re
+import subprocess
 import sys
+import threading
 import time
 
 import torch
@@ -28,12 +38,27 @@ if ROOT not in sys.path:
 
 PEAK = {"bf16": 2500.0, "fp8": 5000.0}   # dense MFMA TFLOP/s, MI355X
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per GEMM1 launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in
-# profiles/ (KiB per dispatch, scaled by the copy-kernel factors 2.0 and 1.0 stated there).
-MEASURED_TRAFFIC_BYTES = {
-    "c3_bf16": int((1.6705e6 * 2.0 + 3.6049e5 * 1.0) * 1024),
-    "c4_fp8": int((9.1226e5 * 2.0 + 3.6486e5 * 1.0) * 1024),
-}
+PROFILE_OF = {"c3_bf16": "moe_forward_c3_bf16_T16384_E64.txt", "c4_fp8": "moe_forward_c4_fp8_T16384_E64.txt"}
+
+
+def measured_traffic_bytes(workload):
+    """HBM-side bytes per GEMM1 launch from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE sections of
+    the workload's summary under profiles/ (KiB per dispatch of the epi=2 ring kernel), scaled by the
+    copy-kernel factors that summary states (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  None if the
+    summary is missing or has no such lines."""
+    name = PROFILE_OF.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return None
+    text = open(path).read()
+    vals = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        m = re.search(r"^\s*gemm_ring\S* fp8=\w+ epi=2\s+" + counter + r"=([0-9.e+]+)\s*$", text, re.M)
+        if not m:
+            return None
+        vals[counter] = float(m.group(1))
+    return int((vals["FETCH_SIZE"] * 2.0 + vals["WRITE_SIZE"] * 1.0) * 1024)
+
 
 WORKLOADS = {
     # name: (T, E, K, D, H, O, kind, dtype, routing)
@@ -187,7 +212,29 @@ def algorithmic_bytes(w, name):
     return None
 
 
-def run_gpu(w, steps, warmup):
+def step_samples(fn, n, stream, flush=None):
+    """Per-step milliseconds from one HIP-event pair per step.  `flush`: a tensor rewritten before
+    every step, outside the event pair, so that the step starts with cold caches."""
+    pairs = []
+    for _ in range(n):
+        if flush is not None:
+            flush.add_(1)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(stream)
+        fn()
+        b.record(stream)
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) for a, b in pairs)
+
+
+def quantiles(samples):
+    n = len(samples)
+    return {"median": round(samples[n // 2], 4), "p95": round(samples[min(n - 1, int(math.ceil(0.95 * n)) - 1)], 4),
+            "min": round(samples[0], 4), "samples": n}
+
+
+def run_gpu(w, steps, warmup, detail=True):
     dev = torch.device("cuda:0")
     inp = make_inputs(w, dev)
     path = GpuPath(w, inp)
@@ -200,12 +247,22 @@ def run_gpu(w, steps, warmup):
         path.step()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / steps
-    # per-kernel launch durations, measured live with events over the same number of launches
+    timing = {}
+    if detail:
+        n = max(steps, 100)
+        timing["hot"] = quantiles(step_samples(path.step, n, stream))
+        flush = torch.zeros(512 << 20, dtype=torch.uint8, device=dev)
+        timing["cold"] = quantiles(step_samples(path.step, max(steps, 30), stream, flush))
+        del flush
+    # per-kernel launch durations, measured live with events: 25 warm-up launches, then max(K, 100)
     path.step()
     per = {}
+    reps = max(steps, 100) if detail else steps
     for name, fn in path.pieces():
+        for _ in range(25 if detail else 1):
+            fn()
         torch.cuda.synchronize()
-        per[name] = time_region(fn, steps, stream)
+        per[name] = time_region(fn, reps, stream)
     f1, f2 = flops_of(w)
     kernels = {}
     for name, ms in per.items():
@@ -222,7 +279,7 @@ def run_gpu(w, steps, warmup):
     lengths = path.r["lengths"]
     stats = {"rows_max": int(lengths.max()), "rows_min": int(lengths.min()),
              "empty_experts": int((lengths == 0).sum())}
-    return ms_step, kernels, stats, (f1, f2)
+    return ms_step, kernels, stats, (f1, f2), timing
 
 
 def cpu_baseline(w, budget_s=12.0):
@@ -231,7 +288,7 @@ def cpu_baseline(w, budget_s=12.0):
     from oracle import layer as o_layer
     from oracle import moe as o_moe
     from oracle import moe_fp8 as o_fp8
-    cores = torch.get_num_threads()
+    cores = torch.get_num_threads()           # the threads the oracle's torch calls actually use
     sample_T = 256
     result = None
     while True:
@@ -270,7 +327,8 @@ def cpu_baseline(w, budget_s=12.0):
         result = {"value": round((f1 + f2) / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                   "sample": f"oracle PyTorch-kernel path, {w['dtype']} emulation, T={sample_T} of {w['T']} tokens "
                             f"(same E/K/D/H, same routing law), median of 3 passes after 1 warm-up, {dt:.2f} s each",
-                  "tokens_per_s": round(sample_T / dt, 1)}
+                  "tokens_per_s": round(sample_T / dt, 1), "torch_num_threads": cores,
+                  "host_logical_cpus": os.cpu_count()}
         if dt * 4 > budget_s or sample_T * 4 > w["T"]:
             return result
         sample_T *= 4
@@ -352,12 +410,151 @@ def run_sgmoe(steps, warmup, tokens):
     return ms_eval, ms_front, ms_train, flops, (T, D, H, E, K)
 
 
-def bench_workload(name, steps, warmup, tokens=None):
+def bench_workload(name, steps, warmup, tokens=None, detail=True):
     w = dict(WORKLOADS[name])
     if tokens:
         w["T"] = tokens
-    ms, kernels, stats, (f1, f2) = run_gpu(w, steps, warmup)
-    return w, ms, kernels, stats, f1 + f2
+    ms, kernels, stats, (f1, f2), timing = run_gpu(w, steps, warmup, detail)
+    return w, ms, kernels, stats, f1 + f2, timing
+
+
+def weight_stream_bytes(w, lengths_nonzero):
+    """Algorithmic HBM bytes of one forward in the weight-streaming regime (few rows per expert):
+    the weights of the experts that have a row, the tokens in and the outputs out."""
+    wb = 1 if w["dtype"] == "fp8" else 2
+    hn = 2 * w["H"] if w["kind"] == "swiglu" else w["H"]
+    return lengths_nonzero * (w["D"] * hn + w["H"] * w["O"]) * wb + w["T"] * w["D"] * 2 + w["T"] * w["O"] * 2
+
+
+def extra_workloads(steps, warmup):
+    """The other configurations of the baseline beside the headline pair, one short entry each:
+    C2 (8 experts, top-2, SiLU MLP) and the 128-expert sweep in bf16 and e4m3 (GB/s of the weight
+    stream up to 512 tokens, TFLOP/s above), plus the one-off weight quantisation of the
+    64-expert configuration (not part of a step)."""
+    out = {}
+    w, ms, kern, stats, fl, _ = bench_workload("c2_bf16", steps, warmup, detail=False)
+    out["c2_bf16"] = {"tokens": w["T"], "ms_per_step": round(ms, 4), "tflops": round(fl / ms / 1e9, 1),
+                      "tokens_per_s": round(w["T"] / ms * 1e3, 1)}
+    for name in ("c5_bf16", "c5_fp8"):
+        sweep = {}
+        for T in (64, 512, 4096, 32768):
+            w, ms, kern, stats, fl, _ = bench_workload(name, steps, warmup, tokens=T, detail=False)
+            entry = {"ms_per_step": round(ms, 4), "tokens_per_s": round(T / ms * 1e3, 1),
+                     "gemm1_ms": kern["gemm1"]["ms"], "gemm2_ms": kern["gemm2"]["ms"]}
+            if T <= 512:
+                touched = w["E"] - stats["empty_experts"]
+                entry["gbs"] = round(weight_stream_bytes(w, touched) / ms / 1e6, 1)
+                entry["frac_hbm"] = round(entry["gbs"] / HBM_PEAK_GBS, 4)
+            else:
+                entry["tflops"] = round(fl / ms / 1e9, 1)
+                entry["frac_mfma"] = round(entry["tflops"] / PEAK["fp8" if w["dtype"] == "fp8" else "bf16"], 4)
+            sweep[str(T)] = entry
+        out[name] = sweep
+        torch.cuda.empty_cache()
+    out["weight_quant_c4"] = weight_quant_rate(WORKLOADS["c4_fp8"], steps)
+    return out
+
+
+def weight_quant_rate(w, steps):
+    """GB/s of the one-off e4m3 quantisation of the expert weights (3 B per element: bf16 in, e4m3 out)."""
+    from fast_moe_amd.kernels import moe_fp8
+    dev = torch.device("cuda:0")
+    E, D, H, O = w["E"], w["D"], w["H"], w["O"]
+    g = torch.Generator(device=dev).manual_seed(2)
+    ws = [(torch.randn(E, H, D, generator=g, device=dev) * D ** -0.5).to(torch.bfloat16).permute(0, 2, 1) for _ in range(2)]
+    ws.append((torch.randn(E, O, H, generator=g, device=dev) * H ** -0.5).to(torch.bfloat16).permute(0, 2, 1))
+    stream = torch.cuda.current_stream(dev)
+
+    def run():
+        for t in ws:
+            moe_fp8.quantize_expert_weights(t)
+
+    run()
+    torch.cuda.synchronize()
+    ms = time_region(run, max(5, steps // 2), stream)
+    nbytes = sum(t.numel() for t in ws) * 3 + sum(t.shape[0] * t.shape[2] for t in ws) * 4
+    return {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+
+class ClockSampler:
+    """Shader clock while the GPU works: `rocm-smi --showclocks` polled from a thread (a child
+    process per sample; this process is not replaced).  The MFMA peak scales with this clock."""
+
+    def __init__(self, period=0.25):
+        self.samples, self.period, self._stop = [], period, threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        while not self._stop.is_set():
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+                m = re.search(r"sclk clock level: \d+: \((\d+)Mhz\)", out)
+                if m:
+                    self.samples.append(int(m.group(1)))
+            except Exception:
+                pass
+            self._stop.wait(self.period)
+
+    def __enter__(self):
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join(timeout=10)
+
+
+def sustained(fn, seconds, sampler_period=0.25):
+    """Runs `fn` back to back for about `seconds` and samples the shader clock meanwhile."""
+    stream = torch.cuda.current_stream()
+    fn()
+    torch.cuda.synchronize()
+    with ClockSampler(sampler_period) as cs:
+        t_end = time.perf_counter() + seconds
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() < t_end:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            n += 20
+        ms = (time.perf_counter() - t0) * 1e3 / n
+    s = sorted(cs.samples[1:] or cs.samples)
+    clock = {"median_mhz": s[len(s) // 2], "min_mhz": s[0], "max_mhz": s[-1], "samples": len(s)} if s else None
+    return ms, clock
+
+
+def sustained_section(w, sample_clock, dense_reference, seconds=3.0):
+    """Each GEMM of the workload run back to back for ~3 s: milliseconds per launch, TFLOP/s, and the
+    shader clock rocm-smi reports meanwhile; with `dense_reference` the vendor's dense GEMM
+    (torch.matmul) on one product of the same FLOPs (R x K x N with the experts' columns side by
+    side) measured the same way.  bf16 workloads only for the dense reference."""
+    dev = torch.device("cuda:0")
+    inp = make_inputs(w, dev)
+    path = GpuPath(w, inp)
+    path.step()
+    f1, f2 = flops_of(w)
+    out = {}
+    for name, fn, fl in (("gemm1", path.gemm1, f1), ("gemm2", path.gemm2, f2)):
+        ms, clock = sustained(fn, seconds)
+        peak = PEAK["fp8" if w["dtype"] == "fp8" else "bf16"]
+        entry = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "sclk": clock}
+        if clock:
+            entry["frac_of_peak_at_clock"] = round(fl / ms / 1e9 / (peak * clock["median_mhz"] / 2400.0), 4)
+        out[name] = entry
+    if dense_reference and w["dtype"] == "bf16":
+        R = w["T"] * w["K"]
+        hn = 2 * w["H"] if w["kind"] == "swiglu" else w["H"]
+        for name, (m, k, n) in (("dense_gemm1", (R, w["D"], hn)), ("dense_gemm2", (R, w["H"], w["O"]))):
+            a = torch.randn(m, k, device=dev).to(torch.bfloat16)
+            b = (torch.randn(n, k, device=dev) * k ** -0.5).to(torch.bfloat16).t()
+            ms, clock = sustained(lambda: torch.matmul(a, b), seconds)
+            fl = 2.0 * m * k * n
+            entry = {"shape_mkn": [m, k, n], "ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "sclk": clock}
+            if clock:
+                entry["frac_of_peak_at_clock"] = round(fl / ms / 1e9 / (PEAK["bf16"] * clock["median_mhz"] / 2400.0), 4)
+            out[name] = entry
+            del a, b
+    return out
 
 
 def main():
@@ -373,6 +570,12 @@ def main():
                     help="time forward + backward of the bf16 SwiGLU workload instead of the forward metric")
     ap.add_argument("--sgmoe", action="store_true",
                     help="time the SGMoE layer (MRN router front-end + experts), forward and training step")
+    ap.add_argument("--sample-clock", action="store_true",
+                    help="run each GEMM of the workload back to back for ~3 s and report the shader clock "
+                         "rocm-smi shows meanwhile (the MFMA peak scales with it)")
+    ap.add_argument("--dense-reference", action="store_true",
+                    help="also time the vendor's dense GEMM (torch.matmul) on the FLOP-equivalent single product "
+                         "of each GEMM of the workload, with the shader clock, for scale")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 512 MiB device copy, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -411,7 +614,7 @@ def main():
                                    f"gradients), T={w['T']}, E={w['E']}, top-{w['K']}, D={w['D']}, H={w['H']}",
                        "flops": "3 x forward GEMM FLOPs"}}))
         return
-    w, ms, kernels, stats, flops = bench_workload(args.workload, args.steps, args.warmup, args.tokens)
+    w, ms, kernels, stats, flops, timing = bench_workload(args.workload, args.steps, args.warmup, args.tokens)
     dt = w["dtype"]
     g1 = kernels["gemm1"]
     line = {
@@ -420,6 +623,11 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if dt == "bf16" else "fp8_e4m3", "data": "synthetic",
         "tokens_per_s": round(w["T"] / ms * 1e3, 1),
+        "timing": {"method": "value: K back-to-back steps between two synchronisations; hot / cold: one HIP-event "
+                             "pair per step, cold = a 512 MiB buffer rewritten before every step; kernels: HIP events "
+                             "over max(K, 100) launches after 25 warm-up launches",
+                   "hot_ms": timing.get("hot"), "cold_ms": timing.get("cold"),
+                   "cold_value": round(flops / timing["cold"]["median"] / 1e9, 2) if timing.get("cold") else None},
         "config": {"workload": f"{args.workload}: {w['kind']} MoE forward, T={w['T']} tokens, E={w['E']} experts, "
                                f"top-{w['K']}, D={w['D']}, H={w['H']}, O={w['O']}, routing={w['routing']}",
                    "tokens": w["T"], "experts": w["E"], "top_k": w["K"], "d_model": w["D"], "hidden": w["H"],
@@ -429,15 +637,18 @@ def main():
                      ("SwiGLU" if w["kind"] == "swiglu" else "SiLU") + " epilogue)",
                      "achieved": g1["tflops"], "peak": PEAK[dt], "unit": "TFLOP/s",
                      "frac": round(g1["tflops"] / PEAK[dt], 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if not args.tokens else None},
+                     "traffic": measured_traffic_bytes(args.workload) if not args.tokens else None},
     }
     if not args.no_extra:
         other = {"c3_bf16": "c4_fp8", "c4_fp8": "c3_bf16"}.get(args.workload)
         if other:
-            w2, ms2, k2, _, fl2 = bench_workload(other, args.steps, args.warmup)
+            w2, ms2, k2, _, fl2, tm2 = bench_workload(other, args.steps, args.warmup)
             line["extra"] = {other: {"value": round(fl2 / ms2 / 1e9, 2), "unit": "TFLOP/s",
                                      "ms_per_step": round(ms2, 4), "tokens_per_s": round(w2["T"] / ms2 * 1e3, 1),
-                                     "kernels": k2}}
+                                     "hot_ms": tm2.get("hot"), "cold_ms": tm2.get("cold"), "kernels": k2}}
+            line["extra"].update(extra_workloads(args.steps, args.warmup))
+    if args.sample_clock or args.dense_reference:
+        line["sustained"] = sustained_section(w, args.sample_clock, args.dense_reference)
     if args.calibrate_copy:      # a kernel of known traffic: 512 MiB read + 512 MiB written
         src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)

@@ -1,6 +1,8 @@
 // fmoe_grouped_gemm: argument checks and kernel selection for the jagged GEMM.
 #include "gemm_kernel.h"
 
+#include <cstdlib>
+
 using namespace fmoe;
 
 namespace fmoe {
@@ -118,6 +120,12 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     const int vec_cols = f32 ? 4 : 8;
     p.k_window = d->k_window;
     p.k_window_multiple = d->k_window ? d->k_window_multiple : 0;
+#ifdef FMOE_TRACE
+    {   // debug builds only: FMOE_TRACE_PTR=<device address in hex> of a zeroed 2 x [grid][32][2][8] uint64 buffer
+        const char* t = getenv("FMOE_TRACE_PTR");
+        p.trace = t ? (uint64_t*)strtoull(t, nullptr, 16) : nullptr;
+    }
+#endif
     p.aux = (uint16_t*)d->aux;
     p.aux2 = (uint16_t*)d->aux2;
     p.aux_stride = d->aux_stride_row;

@@ -75,7 +75,24 @@ struct GemmParams {
     int64_t out_half;
     const uint8_t* a2;                  // second product a2 * b2 summed into the same output, or null
     int k_split;                        // ... whose contraction covers k in [k_split, K)
+#ifdef FMOE_TRACE
+    uint64_t* trace;                    // debug builds: per-tile time stamps of the ring kernel
+#endif
 };
+
+#ifdef FMOE_TRACE
+// Debug builds (-DFMOE_TRACE): wave 0 and wave NW/2 of every block record real-time stamps (100 MHz)
+// per tile into p.trace, two planes of [block][tile < 32][wave group][8]: plane 0 = tile start, end
+// of the main loop, next tile located, epilogue done, shader clock at start and end, K-slices, valid
+// rows; plane 1 = after the first four double steps, before and after the second last one.
+#define FMOE_TRACE_STAMP(slot_)                                                                   \
+    do {                                                                                         \
+        if (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2))                             \
+            tstamp[slot_] = __builtin_amdgcn_s_memrealtime();                                    \
+    } while (0)
+#else
+#define FMOE_TRACE_STAMP(slot_) do {} while (0)
+#endif
 
 constexpr int kDtBf16 = 0, kDtE4m3 = 1, kDtF32 = 2;
 constexpr int kGroupM = 4;   // row tiles per scheduling group
@@ -146,11 +163,16 @@ template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = f
           bool OUT2 = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
-                                              int lane) {
+                                              int lane, uint64_t* ets = nullptr) {
     constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
     constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
     const int khalf = lane >> 5;
     const int64_t bias_row = (int64_t)expert * p.bias_se;
+#ifdef FMOE_TRACE
+#define FMOE_EPI_STAMP(i_) do { if (ets) ets[i_] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define FMOE_EPI_STAMP(i_) do {} while (0)
+#endif
     // Output addresses are a wave-uniform 64-bit base (tile row block, column group: scalar
     // registers and scalar arithmetic) plus one 32-bit per-lane byte offset (the lane's row
     // inside the 32-row block and its 16-byte half): no per-row pointers to keep in vector
@@ -174,6 +196,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         row_ok[fm] = wm * TM + fm * 32 + (lane & 31) < rows_valid;
         rsa[fm] = 1.0f;
     }
+    // per-column reciprocal weight scales of this lane (e4m3): [fn][gp][q][j] <-> column
+    // nq + 8*q + 4*khalf + j with nq = first column of register-quad pair gp of fragment fn
+    float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4];
+    const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
     if (FP8) {
         // the activation scales of this lane's rows: all index loads, then all scale loads (two
         // memory latencies, not two per row block)
@@ -199,8 +225,64 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         }
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) rsa[fm] = p.a_scale[src[fm]];
+        // The weight-scale loads go out right behind the activation-scale loads, before anything
+        // waits for either, so that the two round trips overlap (one memory latency per tile less;
+        // the raw values wait in the registers their reciprocals end up in).
+        constexpr int WCOLS = FN_OUT * 32;          // output columns of this wave
+        if (p.scale_vec && col0 + WCOLS <= p.N) {
+            // the wave's columns lie inside N: the 4 scales of a register quad in one 16-byte load
+            // from a wave-uniform base plus the lane half's 16 bytes plus a constant
+            const float* sb = p.b_scale + ((int64_t)expert * p.N + col0);
+            const float* sb2 = SWIGLU ? p.b2_scale + ((int64_t)expert * p.N + col0) : sb;
+            const int half4 = 4 * khalf;
+            typedef __attribute__((ext_vector_type(4))) float f32x4;
+#pragma unroll
+            for (int fn = 0; fn < FN_OUT; ++fn)
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp)
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const int c = fn * 32 + 16 * gp + 8 * q;
+                        const f32x4 s1 = *reinterpret_cast<const f32x4*>(sb + half4 + c);
+                        f32x4 s2 = s1;
+                        if (SWIGLU) s2 = *reinterpret_cast<const f32x4*>(sb2 + half4 + c);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            rsw[fn][gp][q][j] = s1[j];
+                            rsw2[fn][gp][q][j] = s2[j];
+                        }
+                    }
+        } else {
+            // the last column tile, or scale tensors off a 16-byte boundary: one clamped load a column
+#pragma unroll
+            for (int fn = 0; fn < FN_OUT; ++fn)
+#pragma unroll
+                for (int gp = 0; gp < 2; ++gp)
+#pragma unroll
+                    for (int q = 0; q < 2; ++q)
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
+                            const int nc = n < p.N ? n : p.N - 1;
+                            rsw[fn][gp][q][j] = rsw2[fn][gp][q][j] = p.b_scale[(int64_t)expert * p.N + nc];
+                            if (SWIGLU) rsw2[fn][gp][q][j] = p.b2_scale[(int64_t)expert * p.N + nc];
+                        }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // (v_rcp_f32 is exact on the powers of two the reference's scales are)
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) rsa[fm] = __builtin_amdgcn_rcpf(rsa[fm]);
+#pragma unroll
+        for (int fn = 0; fn < FN_OUT; ++fn)
+#pragma unroll
+            for (int gp = 0; gp < 2; ++gp)
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        rsw[fn][gp][q][j] = __builtin_amdgcn_rcpf(rsw[fn][gp][q][j]);
+                        if (SWIGLU) rsw2[fn][gp][q][j] = __builtin_amdgcn_rcpf(rsw2[fn][gp][q][j]);
+                    }
     }
     // the bias-free form (FastMoE's SwiGLU experts, every fp8 call without bias) skips the adds
     auto run = [&](auto has_bias_c, auto has_aux_c) {
@@ -208,10 +290,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         constexpr bool HAS_AUX = SWIGLU && decltype(has_aux_c)::value;   // keep the pre-activations (training)
         constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && !FP8 && FN_OUT == 2;   // (the e4m3 kernels have no registers to spare for it)
         constexpr bool PAIRS = FP8 && !SWIGLU;      // the cheap half of it, per 16-column group (measured: no gain on the SwiGLU epilogues)
-        // per-column epilogue constants of this lane: [fn][gp][q][j] <-> column nq + 8*q + 4*khalf + j
-        // with nq = first column of register-quad pair gp of fragment fn
-        float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4], bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
-        const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
+        // per-column biases of this lane, indexed like rsw
+        float bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
         // with a bias, at least one of the two pointers is set: both loads go through a valid
         // pointer and a select drops the value of a missing one (a branch per load would make
         // every load wait for the one before)
@@ -227,12 +307,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     for (int j = 0; j < 4; ++j) {
                         const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf + j;
                         const int nc = n < p.N ? n : p.N - 1;
-                        // (v_rcp_f32 is exact on the powers of two the reference's scales are)
-                        rsw[fn][gp][q][j] = rsw2[fn][gp][q][j] = 1.0f;
-                        if (FP8 && !p.scale_vec) {
-                            rsw[fn][gp][q][j] = __builtin_amdgcn_rcpf(p.b_scale[(int64_t)expert * p.N + nc]);
-                            if (SWIGLU) rsw2[fn][gp][q][j] = __builtin_amdgcn_rcpf(p.b2_scale[(int64_t)expert * p.N + nc]);
-                        }
                         bv[fn][gp][q][j] = bv2[fn][gp][q][j] = 0.0f;
                         if (HAS_BIAS) {
                             const float a = bf16_bits_to_f32(bias_a[bias_row + nc]);
@@ -243,32 +317,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                             bv2[fn][gp][q][j] = p.bias2 ? b : 0.0f;
                         }
                     }
-        if (FP8 && p.scale_vec) {
-            // the 4 scales of a register quad in one 16-byte load (a quad that begins past the
-            // last column reads the last 4 scales instead: its columns are never stored)
-#pragma unroll
-            for (int fn = 0; fn < FN_OUT; ++fn)
-#pragma unroll
-                for (int gp = 0; gp < 2; ++gp)
-#pragma unroll
-                    for (int q = 0; q < 2; ++q) {
-                        const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf;
-                        const int64_t at = (int64_t)expert * p.N + (n + 3 < p.N ? n : p.N - 4);
-                        typedef __attribute__((ext_vector_type(4))) float f32x4;
-                        const f32x4 s1 = *reinterpret_cast<const f32x4*>(p.b_scale + at);
-                        f32x4 s2 = s1;
-                        if (SWIGLU) s2 = *reinterpret_cast<const f32x4*>(p.b2_scale + at);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            rsw[fn][gp][q][j] = __builtin_amdgcn_rcpf(s1[j]);
-                            if (SWIGLU) rsw2[fn][gp][q][j] = __builtin_amdgcn_rcpf(s2[j]);
-                        }
-                    }
-        }
         __builtin_amdgcn_sched_barrier(0);
+        FMOE_EPI_STAMP(0);
         // rows outermost: the stores that complete a row's 128-byte line follow each other
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
+            if (fm > 0) FMOE_EPI_STAMP(fm);
             if constexpr (QUAD) {
                 // The store unit merges what ADJACENT lanes write: a lane and its partner 32 lanes
                 // away cost two requests even for neighbouring bytes, four adjacent lanes on 64
@@ -508,6 +562,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         // compiler's count, and the wait for it lands where its register is next written:
         // inside the caller's steady-state loop, where it would also drain the LDS-DMA stream,
         // which the compiler cannot see, on every iteration.
+        FMOE_EPI_STAMP(FM);
         wait_vmcnt<FM * FN_OUT * 2 * (HAS_AUX ? 3 : 1)>();      // (the scalar-store path issues more)
     };
     if (SWIGLU && p.aux) {
@@ -1472,6 +1527,11 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             for (int j = 0; j < FM; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+#ifdef FMOE_TRACE
+        uint64_t tstamp[18] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        FMOE_TRACE_STAMP(0);
+        if (p.trace) tstamp[4] = __builtin_amdgcn_s_memtime();
+#endif
         if (EARLY_ROWS) rows_to_offsets(ridx_next, xoff_next);      // the tile after this one
         else if (tile_i > 0) prefetch_next();
 
@@ -1655,10 +1715,17 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             // the last two double steps hold the end of an XTR tile's window and mask it
             auto tile_steps = [&](auto half_c) {
                 const int tile_kt = KWIN ? cur.kt : KT;
-                for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{}, std::false_type{});
+                for (int kt = 0; kt < tile_kt - 4; kt += 2) {
+                    double_step(half_c, std::false_type{}, std::false_type{});
+#ifdef FMOE_TRACE
+                    if (kt < 8) FMOE_TRACE_STAMP(6 + kt / 2);
+#endif
+                }
+                FMOE_TRACE_STAMP(10);
                 enter_next();
                 ikt = 0;
                 double_step(half_c, std::false_type{}, std::true_type{});
+                FMOE_TRACE_STAMP(11);
                 double_step(half_c, std::true_type{}, std::true_type{});
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
@@ -1757,10 +1824,17 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 // counts as pending from the tile's set-up or the last epilogue (spill reloads,
                 // the row-index loads).  Left pending, their waits land inside the loop, where
                 // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
-                for (int kt = 0; kt < tile_kt - 4; kt += 2) double_step(half_c, std::false_type{});
+                for (int kt = 0; kt < tile_kt - 4; kt += 2) {
+                    double_step(half_c, std::false_type{});
+#ifdef FMOE_TRACE
+                    if (kt < 8) FMOE_TRACE_STAMP(6 + kt / 2);
+#endif
+                }
+                FMOE_TRACE_STAMP(10);
                 enter_next();
                 ikt = 0;
                 double_step(half_c, std::false_type{});
+                FMOE_TRACE_STAMP(11);
                 double_step(half_c, std::true_type{});
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
@@ -1790,12 +1864,37 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             wait_vmcnt<L>();
             landed = issued - 2;
         }
+        FMOE_TRACE_STAMP(1);
         const TileInfo done = cur;
         cur = nxt;          // valid when another tile follows
         if (EARLY_ROWS) prefetch_next();    // nxt: the tile after that one; its row indices arrive during the epilogue
+        FMOE_TRACE_STAMP(2);
 
+#ifdef FMOE_TRACE
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(
+            p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane,
+            (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2)) ? tstamp + 12 : nullptr);
+#else
         gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                                 done.rows_valid, wm, wn, lane);
+#endif
+#ifdef FMOE_TRACE
+        FMOE_TRACE_STAMP(3);
+        if (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2) && lane == 0) {
+            tstamp[5] = __builtin_amdgcn_s_memtime();
+            uint64_t* dst = p.trace + (((int64_t)blockIdx.x * 32 + tile_i) * 2 + (wave != 0)) * 8;
+#pragma unroll
+            for (int j = 0; j < 6; ++j) dst[j] = tstamp[j];
+            dst[6] = (uint64_t)KT;
+            dst[7] = (uint64_t)done.rows_valid;
+            uint64_t* dst2 = p.trace + (int64_t)gridDim.x * 32 * 2 * 8 + (((int64_t)blockIdx.x * 32 + tile_i) * 2 + (wave != 0)) * 8;
+#pragma unroll
+            for (int j = 0; j < 6; ++j) dst2[j] = tstamp[6 + j];
+            uint64_t* dst3 = dst2 + (int64_t)gridDim.x * 32 * 2 * 8;
+#pragma unroll
+            for (int j = 0; j < 6; ++j) dst3[j] = tstamp[12 + j];
+        }
+#endif
     }
     wait_vmcnt<0>();    // nothing may still be on its way into this block's LDS when it ends
 }
