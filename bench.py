@@ -129,7 +129,8 @@ class GpuPath:
 
     # --- the pieces
     def route(self):
-        self.r = self.ops.route_topk(self.inp["scores"], self.w["K"])
+        # (the routing tensors of the previous step are written in place: a serving loop keeps them)
+        self.r = self.ops.route_topk(self.inp["scores"], self.w["K"], out=getattr(self, "r", None))
         return self.r
 
     def quant_tokens(self):

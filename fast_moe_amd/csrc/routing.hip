@@ -4,14 +4,15 @@
 // function of the selected ids (a stable counting sort), so they are
 // reproducible bit for bit.
 //
-// Pipeline (4 launches on one stream, no host synchronisation):
-//   1. topk_kernel     rank-by-counting selection, one token per LPT lanes
-//   2. hist_kernel     one wave per chunk of tokens: LDS histogram -> chunk_hist[c][e]
-//   3. scan_kernel     one block per expert: exclusive scan of chunk_hist over the
-//                      chunks (in place, wave scans), lengths[e]
-//   4. scatter_kernel  one wave per chunk: offsets = wave scan of lengths, then a
-//                      wave-level match/rank gives each position its slot inside
-//                      its expert segment
+// Two launches on one stream, no host synchronisation.  The tokens are cut into up to 256
+// chunks (one block of 4 waves each, a wave owns a contiguous quarter of its chunk):
+//   1. topk_hist_kernel (or compact_hist_kernel for caller-supplied ids): selection by rank
+//      counting, one token per LPT lanes; every wave counts the experts of its tokens in LDS ->
+//      sub_hist[chunk][wave][e], tot_hist[chunk][e]
+//   2. scan_scatter_kernel: every block sums tot_hist over the chunks before it (and over all
+//      chunks: lengths; wave scan over the experts: offsets), every wave adds the counts of
+//      the waves before it in its chunk and then places its positions: a wave-level
+//      match/rank gives each position its slot inside its expert segment
 #include "common.h"
 
 #include <mutex>
@@ -19,28 +20,57 @@
 namespace fmoe {
 namespace {
 
-constexpr int kMaxChunks = 512;
+constexpr int kMaxChunks = 256;
+constexpr int kMaxRouteWaves = 16;
+// waves per block of both kernels: 16 while the per-wave expert tables fit LDS comfortably
+inline int route_waves(int E) { return E <= 256 ? 16 : 4; }
 constexpr uint16_t kBadExpert = 0xFFFF;
 
 struct RoutePlan {
-    int64_t tokens_per_chunk;
+    int64_t tokens_per_wave;
     int num_chunks;
+    int wpb;                // waves per block
     size_t compact_bytes;   // uint16 expert id per routed position
-    size_t hist_bytes;      // int32 [num_chunks][E]
+    size_t sub_bytes;       // int32 [num_chunks][wpb][E]
+    size_t tot_bytes;       // int32 [num_chunks][E]
+    size_t bad_bytes;       // int32 [num_chunks] out-of-range ids per chunk
     size_t total_bytes;
 };
 
 RoutePlan make_plan(int64_t T, int E, int K) {
     RoutePlan p;
-    p.tokens_per_chunk = (T + kMaxChunks - 1) / kMaxChunks;
-    if (p.tokens_per_chunk < 1) p.tokens_per_chunk = 1;
-    p.num_chunks = (int)((T + p.tokens_per_chunk - 1) / p.tokens_per_chunk);
+    const int kRouteWaves = route_waves(E);
+    p.wpb = kRouteWaves;
+    const int64_t waves = (int64_t)kMaxChunks * kRouteWaves;
+    p.tokens_per_wave = (T + waves - 1) / waves;
+    if (p.tokens_per_wave < 1) p.tokens_per_wave = 1;
+    const int64_t per_chunk = p.tokens_per_wave * kRouteWaves;
+    p.num_chunks = (int)((T + per_chunk - 1) / per_chunk);
     if (p.num_chunks < 1) p.num_chunks = 1;
-    size_t compact = (size_t)T * (size_t)K * sizeof(uint16_t);
-    p.compact_bytes = (compact + 255) & ~(size_t)255;
-    p.hist_bytes = ((size_t)p.num_chunks * (size_t)E * sizeof(int32_t) + 255) & ~(size_t)255;
-    p.total_bytes = p.compact_bytes + p.hist_bytes + 256;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    p.compact_bytes = up((size_t)T * (size_t)K * sizeof(uint16_t));
+    p.sub_bytes = up((size_t)p.num_chunks * kRouteWaves * (size_t)E * sizeof(int32_t));
+    p.tot_bytes = up((size_t)p.num_chunks * (size_t)E * sizeof(int32_t));
+    p.bad_bytes = up((size_t)p.num_chunks * sizeof(int32_t));
+    p.total_bytes = p.compact_bytes + p.sub_bytes + p.tot_bytes + p.bad_bytes + 256;
     return p;
+}
+
+struct RouteScratch {
+    uint16_t* compact;
+    int32_t* sub_hist;
+    int32_t* tot_hist;
+    int32_t* bad_part;
+};
+
+RouteScratch carve(void* workspace, const RoutePlan& plan) {
+    char* w = (char*)workspace;
+    RouteScratch r;
+    r.compact = (uint16_t*)w;
+    r.sub_hist = (int32_t*)(w + plan.compact_bytes);
+    r.tot_hist = (int32_t*)(w + plan.compact_bytes + plan.sub_bytes);
+    r.bad_part = (int32_t*)(w + plan.compact_bytes + plan.sub_bytes + plan.tot_bytes);
+    return r;
 }
 
 template <typename T>
@@ -74,225 +104,349 @@ __device__ __forceinline__ uint32_t order_key(float v) {
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
-// One token per LPT lanes, VPL scores per lane (expert id = v*LPT + sub).  The
-// rank of a score is the number of scores that beat it (greater key, or equal key with
-// a lower expert id); rank < K selects it and is its slot.
-template <typename T, int LPT, int VPL>
-__global__ __launch_bounds__(256) void topk_kernel(const T* __restrict__ scores, int64_t num_tokens,
-                                                   int E, int K, int renorm,
-                                                   int64_t* __restrict__ topk_idx,
-                                                   T* __restrict__ gates,
-                                                   uint16_t* __restrict__ compact) {
-    constexpr int TPW = kWave / LPT;          // tokens per wave
-    constexpr int WPB = 256 / kWave;
+// Largest value over each group of LPT (8 or 16) consecutive lanes, in every lane of the group:
+// butterfly steps on the DPP network inside a row of 16 lanes (quad permutes, mirrors).
+template <int LPT>
+__device__ __forceinline__ uint32_t group_max_u32(uint32_t v) {
+    static_assert(LPT == 8 || LPT == 16, "a group is half a DPP row or a whole one");
+#define FMOE_DPP_MAX(ctrl) v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ctrl, 0xF, 0xF, false))
+    FMOE_DPP_MAX(0xB1);      // quad_perm [1,0,3,2]
+    FMOE_DPP_MAX(0x4E);      // quad_perm [2,3,0,1]
+    FMOE_DPP_MAX(0x141);     // row_half_mirror
+    if (LPT == 16) FMOE_DPP_MAX(0x140);     // row_mirror
+#undef FMOE_DPP_MAX
+    return v;
+}
+
+// Orders this wave's LDS accesses for the compiler.  The hardware runs a wave's LDS instructions in
+// order, and the regions touched between two of these belong to one wave: no block barrier needed.
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// One token per LPT lanes (8 or 16: a token's lanes sit in one DPP row), VPL scores per lane
+// (expert id = v*LPT + sub).  K rounds of "largest remaining key, lowest expert id among equal
+// keys", each two group maxima on the DPP network; the round is the slot (descending score,
+// ties -> lower expert id).
+template <typename T, int LPT, int VPL, int WPB>
+__global__ __launch_bounds__(WPB * kWave) void topk_hist_kernel(const T* __restrict__ scores, int64_t num_tokens,
+                                                        int E, int K, int renorm, int64_t tokens_per_wave,
+                                                        int64_t* __restrict__ topk_idx,
+                                                        T* __restrict__ gates,
+                                                        uint16_t* __restrict__ compact,
+                                                        int32_t* __restrict__ sub_hist,
+                                                        int32_t* __restrict__ tot_hist) {
+    constexpr int TPW = kWave / LPT;          // tokens per wave and pass
+    constexpr int NT = WPB * kWave;
     __shared__ float s_sel[WPB][TPW][64];     // selected scores by slot (K <= 64)
+    extern __shared__ int32_t s_hist[];       // [WPB][E] experts chosen by this wave's tokens
     const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
     const int sub = lane % LPT;
     const int grp = lane / LPT;
-    const int64_t t = ((int64_t)blockIdx.x * WPB + wave) * TPW + grp;
-    const bool live = t < num_tokens;
-
-    float my[VPL];
+    for (int i = threadIdx.x; i < WPB * E; i += NT) s_hist[i] = 0;
+    __syncthreads();
+    // this wave's tokens: a contiguous range, TPW of them per pass; every wave of the grid makes
+    // the same number of passes (the block-wide barriers below sit inside the loop)
+    const int64_t w_begin = ((int64_t)blockIdx.x * WPB + wave) * tokens_per_wave;
+    int64_t w_end = w_begin + tokens_per_wave;
+    if (w_end > num_tokens) w_end = num_tokens;
+    const int64_t passes = (tokens_per_wave + TPW - 1) / TPW;
     const float ninf = -__builtin_inff();
+    // the scores of the next pass are fetched while this one is ranked (as long as registers allow)
+    constexpr bool AHEAD = VPL <= 8;
+    float ahead[AHEAD ? VPL : 1];
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
+    for (int v = 0; v < (AHEAD ? VPL : 0); ++v) {
         const int e = v * LPT + sub;
-        my[v] = (live && e < E) ? load_score<T>(scores + t * E + e) : ninf;
+        const int64_t t0 = w_begin + grp;
+        ahead[v] = (t0 < w_end && e < E) ? load_score<T>(scores + t0 * E + e) : ninf;
     }
-    // modes 2 and 3: the inputs are logits; they are L2-normalised over the experts first
-    // (F.normalize: l / max(||l||, 1e-12), rounded to the logits' dtype), and it is the
-    // normalised values that are ranked: rounding can tie values that differed before
-    if (renorm >= 2) {
-        float sq = 0.0f;
+    for (int64_t pass = 0; pass < passes; ++pass) {
+        const int64_t t = w_begin + pass * TPW + grp;
+        const bool live = t < w_end;
+
+        float my[VPL];
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
             const int e = v * LPT + sub;
-            if (live && e < E) sq += my[v] * my[v];
+            if (AHEAD) {
+                my[v] = ahead[v];
+                const int64_t tn = t + TPW;
+                ahead[v] = (tn < w_end && e < E) ? load_score<T>(scores + tn * E + e) : ninf;
+            } else {
+                my[v] = (live && e < E) ? load_score<T>(scores + t * E + e) : ninf;
+            }
         }
-#pragma unroll
-        for (int o = LPT / 2; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, kWave);
-        const float norm = fmaxf(round_to<T>(sqrtf(sq)), 1e-12f);
-#pragma unroll
-        for (int v = 0; v < VPL; ++v) {
-            const int e = v * LPT + sub;
-            if (live && e < E) my[v] = round_to<T>(my[v] / norm);
-        }
-    }
-    int rank[VPL];
-    uint32_t key[VPL];
-#pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-        rank[v] = 0;
-        key[v] = order_key(my[v]);
-    }
-#pragma unroll
-    for (int u = 0; u < VPL; ++u) {
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) {
-            // a full wave per token: the broadcast lane is a compile-time constant (v_readlane)
-            const uint32_t other = LPT == kWave ? (uint32_t)__builtin_amdgcn_readlane((int)key[u], i)
-                                                : (uint32_t)__shfl((int)key[u], grp * LPT + i, kWave);
-            const int oe = u * LPT + i;
+        // modes 2 and 3: the inputs are logits; they are L2-normalised over the experts first
+        // (F.normalize: l / max(||l||, 1e-12), rounded to the logits' dtype), and it is the
+        // normalised values that are ranked: rounding can tie values that differed before
+        if (renorm >= 2) {
+            float sq = 0.0f;
 #pragma unroll
             for (int v = 0; v < VPL; ++v) {
                 const int e = v * LPT + sub;
-                rank[v] += (other > key[v] || (other == key[v] && oe < e)) ? 1 : 0;
+                if (live && e < E) sq += my[v] * my[v];
+            }
+#pragma unroll
+            for (int o = LPT / 2; o >= 1; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+            const float norm = fmaxf(round_to<T>(sqrtf(sq)), 1e-12f);
+#pragma unroll
+            for (int v = 0; v < VPL; ++v) {
+                const int e = v * LPT + sub;
+                if (live && e < E) my[v] = round_to<T>(my[v] / norm);
             }
         }
-    }
+        int rank[VPL];
+        uint32_t work[VPL];
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-        const int e = v * LPT + sub;
-        if (live && e < E && rank[v] < K) s_sel[wave][grp][rank[v]] = my[v];
-    }
-    // gates of modes 2 and 3: softmax of the normalised logits over all experts (2) or over
-    // the K selected ones (3)
-    float soft_sum = 0.0f;
-    __syncthreads();
-    if (renorm == 2) {
-        // the largest normalised logit is slot 0; exp(n_i - n_max) summed over all experts
-        const float nmax = live ? s_sel[wave][grp][0] : 0.0f;
+        for (int v = 0; v < VPL; ++v) {
+            rank[v] = K;                                                   // not selected
+            // (a key is never 0: -inf maps to 0x007fffff; 0 marks "taken" and the lanes past E)
+            work[v] = (live && v * LPT + sub < E) ? order_key(my[v]) : 0u;
+        }
+        for (int r = 0; r < K; ++r) {
+            uint32_t best = work[0];
+            int bv = 0;
+#pragma unroll
+            for (int v = 1; v < VPL; ++v)
+                if (work[v] > best) {                  // strictly: equal keys keep the lower expert id
+                    best = work[v];
+                    bv = v;
+                }
+            const uint32_t top = group_max_u32<LPT>(best);
+            const uint32_t cand = best == top ? 0x3FFu - (uint32_t)(bv * LPT + sub) : 0u;
+            const int win = (int)(0x3FFu - group_max_u32<LPT>(cand));     // this round's winner in the group
+#pragma unroll
+            for (int v = 0; v < VPL; ++v)
+                if (v * LPT + sub == win) {
+                    rank[v] = r;
+                    work[v] = 0u;
+                }
+        }
 #pragma unroll
         for (int v = 0; v < VPL; ++v) {
             const int e = v * LPT + sub;
-            if (live && e < E) soft_sum += expf(my[v] - nmax);
+            if (live && e < E && rank[v] < K) s_sel[wave][grp][rank[v]] = my[v];
         }
+        // gates of modes 2 and 3: softmax of the normalised logits over all experts (2) or over
+        // the K selected ones (3)
+        float soft_sum = 0.0f;
+        wave_lds_fence();
+        if (renorm == 2) {
+            // the largest normalised logit is slot 0; exp(n_i - n_max) summed over all experts
+            const float nmax0 = live ? s_sel[wave][grp][0] : 0.0f;
 #pragma unroll
-        for (int o = LPT / 2; o >= 1; o >>= 1) soft_sum += __shfl_xor(soft_sum, o, kWave);
-    }
-    if (!live) return;
-    float denom = 1.0f;
-    if (renorm == 1) {
-        float s = 0.0f;
-        for (int j = 0; j < K; ++j) s = s + fabsf(s_sel[wave][grp][j]);   // slot order
-        // (clamp_min keeps a NaN norm, fmaxf would drop it)
-        denom = s != s ? s : fmaxf(round_to<T>(s), round_to<T>(1e-12f));
-    }
-    float nmax = 0.0f;
-    if (renorm >= 2) {
-        nmax = s_sel[wave][grp][0];
-        if (renorm == 3) {
-            soft_sum = 0.0f;
-            for (int j = 0; j < K; ++j) soft_sum += expf(s_sel[wave][grp][j] - nmax);
-        }
-    }
+            for (int v = 0; v < VPL; ++v) {
+                const int e = v * LPT + sub;
+                if (live && e < E) soft_sum += expf(my[v] - nmax0);
+            }
 #pragma unroll
-    for (int v = 0; v < VPL; ++v) {
-        const int e = v * LPT + sub;
-        if (e < E && rank[v] < K) {
-            const int64_t p = t * K + rank[v];
-            topk_idx[p] = e;
-            compact[p] = (uint16_t)e;
-            float g = my[v];
-            if (renorm == 1) g = round_to<T>(my[v] / denom);
-            else if (renorm >= 2) g = round_to<T>(expf(my[v] - nmax) / soft_sum);
-            store_score<T>(gates + p, g);
+            for (int o = LPT / 2; o >= 1; o >>= 1) soft_sum += __shfl_xor(soft_sum, o, kWave);
         }
-    }
-}
-
-// Expert ids supplied by the caller (int64): narrow to the compact form, flag
-// out-of-range ids.
-__global__ __launch_bounds__(256) void compact_kernel(const int64_t* __restrict__ topk_idx, int64_t n,
-                                                      int E, uint16_t* __restrict__ compact,
-                                                      int64_t* __restrict__ bad_count) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const int64_t e = topk_idx[i];
-    const bool ok = e >= 0 && e < E;
-    compact[i] = ok ? (uint16_t)e : kBadExpert;
-    if (!ok && bad_count) atomicAdd((unsigned long long*)bad_count, 1ull);
-}
-
-__global__ void zero_i64_kernel(int64_t* p) { *p = 0; }
-
-// One wave per chunk of tokens; counts are integers, so LDS atomics are exact.
-__global__ __launch_bounds__(kWave) void hist_kernel(const uint16_t* __restrict__ compact,
-                                                     int64_t total_pos, int64_t pos_per_chunk, int E,
-                                                     int32_t* __restrict__ chunk_hist) {
-    extern __shared__ int32_t s_cnt[];
-    const int c = blockIdx.x;
-    for (int e = threadIdx.x; e < E; e += kWave) s_cnt[e] = 0;
-    __syncthreads();
-    const int64_t begin = (int64_t)c * pos_per_chunk;
-    int64_t end = begin + pos_per_chunk;
-    if (end > total_pos) end = total_pos;
-    for (int64_t p = begin + threadIdx.x; p < end; p += kWave) {
-        const uint16_t e = compact[p];
-        if (e != kBadExpert) atomicAdd(&s_cnt[e], 1);
+        if (live) {
+            float denom = 1.0f;
+            if (renorm == 1) {
+                float s = 0.0f;
+                for (int j = 0; j < K; ++j) s = s + fabsf(s_sel[wave][grp][j]);   // slot order
+                // (clamp_min keeps a NaN norm, fmaxf would drop it)
+                denom = s != s ? s : fmaxf(round_to<T>(s), round_to<T>(1e-12f));
+            }
+            float nmax = 0.0f;
+            if (renorm >= 2) {
+                nmax = s_sel[wave][grp][0];
+                if (renorm == 3) {
+                    soft_sum = 0.0f;
+                    for (int j = 0; j < K; ++j) soft_sum += expf(s_sel[wave][grp][j] - nmax);
+                }
+            }
+#pragma unroll
+            for (int v = 0; v < VPL; ++v) {
+                const int e = v * LPT + sub;
+                if (e < E && rank[v] < K) {
+                    const int64_t p = t * K + rank[v];
+                    topk_idx[p] = e;
+                    compact[p] = (uint16_t)e;
+                    atomicAdd(&s_hist[wave * E + e], 1);      // integer counts in LDS: exact
+                    float g = my[v];
+                    if (renorm == 1) g = round_to<T>(my[v] / denom);
+                    else if (renorm >= 2) g = round_to<T>(expf(my[v] - nmax) / soft_sum);
+                    store_score<T>(gates + p, g);
+                }
+            }
+        }
+        wave_lds_fence();       // s_sel is rewritten by the next pass
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < E; e += kWave) chunk_hist[(int64_t)c * E + e] = s_cnt[e];
+    for (int i = threadIdx.x; i < WPB * E; i += NT) sub_hist[(int64_t)blockIdx.x * WPB * E + i] = s_hist[i];
+    for (int e = threadIdx.x; e < E; e += NT) {
+        int32_t tot = 0;
+#pragma unroll
+        for (int w = 0; w < WPB; ++w) tot += s_hist[w * E + e];
+        tot_hist[(int64_t)blockIdx.x * E + e] = tot;
+    }
 }
 
-// One block per expert: exclusive scan of that expert's counts over the chunks (in place)
-// and its total.  256 threads, two chunks per thread (num_chunks <= 512).
-__global__ __launch_bounds__(256) void scan_kernel(int32_t* __restrict__ chunk_hist, int num_chunks, int E,
-                                                   int64_t* __restrict__ lengths) {
-    __shared__ int32_t s_wave[4];
-    const int e = blockIdx.x;
-    const int c0 = threadIdx.x * 2, c1 = c0 + 1;
-    const int32_t v0 = c0 < num_chunks ? chunk_hist[(int64_t)c0 * E + e] : 0;
-    const int32_t v1 = c1 < num_chunks ? chunk_hist[(int64_t)c1 * E + e] : 0;
-    const int inc = wave_inclusive_scan((int)(v0 + v1));
+// Expert ids supplied by the caller (int64): narrow to the compact form, count them per wave
+// and chunk as above, count the out-of-range ids of the chunk.
+__global__ __launch_bounds__(1024) void compact_hist_kernel(const int64_t* __restrict__ topk_idx,
+                                                            int64_t num_tokens, int E, int K,
+                                                            int64_t tokens_per_wave,
+                                                            uint16_t* __restrict__ compact,
+                                                            int32_t* __restrict__ sub_hist,
+                                                            int32_t* __restrict__ tot_hist,
+                                                            int32_t* __restrict__ bad_part) {
+    const int WPB = blockDim.x / kWave, NT = blockDim.x;
+    extern __shared__ int32_t s_hist[];       // [WPB][E], then [WPB] bad counts
+    int32_t* s_bad = s_hist + WPB * E;
+    const int lane = lane_id();
     const int wave = threadIdx.x / kWave;
-    if (lane_id() == kWave - 1) s_wave[wave] = inc;
+    for (int i = threadIdx.x; i < WPB * E + WPB; i += NT) s_hist[i] = 0;
     __syncthreads();
-    int base = 0;
-    for (int w = 0; w < wave; ++w) base += s_wave[w];
-    const int excl = base + inc - (v0 + v1);
-    if (c0 < num_chunks) chunk_hist[(int64_t)c0 * E + e] = excl;
-    if (c1 < num_chunks) chunk_hist[(int64_t)c1 * E + e] = excl + v0;
-    if (threadIdx.x == 255) lengths[e] = base + inc;
+    const int64_t w_begin = ((int64_t)blockIdx.x * WPB + wave) * tokens_per_wave;
+    int64_t w_end = w_begin + tokens_per_wave;
+    if (w_end > num_tokens) w_end = num_tokens;
+    int bad = 0;
+    for (int64_t p = w_begin * K + lane; p < w_end * K; p += kWave) {
+        const int64_t e = topk_idx[p];
+        const bool ok = e >= 0 && e < E;
+        compact[p] = ok ? (uint16_t)e : kBadExpert;
+        if (ok) atomicAdd(&s_hist[wave * E + (int)e], 1);
+        else ++bad;
+    }
+    if (bad) atomicAdd(&s_bad[wave], bad);
+    __syncthreads();
+    for (int i = threadIdx.x; i < WPB * E; i += NT) sub_hist[(int64_t)blockIdx.x * WPB * E + i] = s_hist[i];
+    for (int e = threadIdx.x; e < E; e += NT) {
+        int32_t tot = 0;
+        for (int w = 0; w < WPB; ++w) tot += s_hist[w * E + e];
+        tot_hist[(int64_t)blockIdx.x * E + e] = tot;
+    }
+    if (threadIdx.x == 0) {
+        int32_t b = 0;
+        for (int w = 0; w < WPB; ++w) b += s_bad[w];
+        bad_part[blockIdx.x] = b;
+    }
 }
 
-// One wave per chunk.  Each iteration takes TPI = 64/K whole tokens, lane i <->
-// position chunk_begin + it*TPI*K + i, so the K slots of a token sit in one
-// iteration.  s_next[e] is the next free slot of expert e for this chunk.
-__global__ __launch_bounds__(kWave) void scatter_kernel(const uint16_t* __restrict__ compact,
-                                                        int64_t num_tokens, int64_t tokens_per_chunk,
-                                                        int E, int K, int ebits,
-                                                        const int32_t* __restrict__ chunk_base,
-                                                        const int64_t* __restrict__ lengths,
-                                                        int64_t* __restrict__ offsets,
-                                                        int64_t* __restrict__ gate_index,
-                                                        int64_t* __restrict__ token_index,
-                                                        int64_t* __restrict__ reverse_index) {
-    extern __shared__ int32_t s_next[];
+// Block = chunk, 4 or 16 waves.  Phase 1: per expert, the rows of all chunks (lengths) and of the chunks
+// before this one.  Phase 2: wave scan over the experts = offsets.  Phase 3: every wave starts
+// from offsets + rows of earlier chunks + rows of the earlier waves of its chunk and places its
+// positions.  Each pass takes TPI = 64/K whole tokens, lane i <-> position begin + pass*TPI*K + i,
+// so the K slots of a token sit in one pass.  s_next[e] is the next free slot of expert e.
+__global__ __launch_bounds__(1024) void scan_scatter_kernel(const uint16_t* __restrict__ compact,
+                                                           int64_t num_tokens, int64_t tokens_per_wave,
+                                                           int E, int K, int ebits, int num_chunks,
+                                                           const int32_t* __restrict__ sub_hist,
+                                                           const int32_t* __restrict__ tot_hist,
+                                                           const int32_t* __restrict__ bad_part,
+                                                           int64_t* __restrict__ lengths,
+                                                           int64_t* __restrict__ offsets,
+                                                           int64_t* __restrict__ gate_index,
+                                                           int64_t* __restrict__ token_index,
+                                                           int64_t* __restrict__ reverse_index,
+                                                           int64_t* __restrict__ bad_count) {
+    const int WPB = blockDim.x / kWave;
+    extern __shared__ int32_t smem[];
+    int32_t* s_tot = smem;                    // [WPB][E] partial sums over a share of the chunks
+    int32_t* s_bef = smem + WPB * E;          // [WPB][E] ... restricted to the chunks before this one
+    int32_t* s_base = smem + 2 * WPB * E;     // [E] first slot of this chunk's rows of expert e
+    int32_t* s_next = smem + 2 * WPB * E + E; // [WPB][E]: first this chunk's counts per wave, then the next free slots
     const int c = blockIdx.x;
-    const int lane = threadIdx.x;
-    {   // exclusive prefix of lengths over the experts = offsets (wave scan); chunk 0 publishes it
+    const int lane = lane_id();
+    const int wave = threadIdx.x / kWave;
+    {   // phase 1: wave w sums chunks [w * q, (w + 1) * q)
+        const int q = (num_chunks + WPB - 1) / WPB;
+        const int c_lo = wave * q, c_hi = (wave + 1) * q < num_chunks ? (wave + 1) * q : num_chunks;
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int e = e0 + lane;
+            int32_t tot = 0, bef = 0;
+            if (e < E) {
+                // (this wave's own counts of the chunk ride along with the first loads)
+                s_next[wave * E + e] = sub_hist[((int64_t)c * WPB + wave) * E + e];
+#pragma unroll 8
+                for (int cc = c_lo; cc < c_hi; ++cc) {
+                    const int32_t v = tot_hist[(int64_t)cc * E + e];
+                    tot += v;
+                    bef += cc < c ? v : 0;
+                }
+                s_tot[wave * E + e] = tot;
+                s_bef[wave * E + e] = bef;
+            }
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {    // phase 2: exclusive prefix of the lengths over the experts; chunk 0 publishes
         long long run = 0;
         for (int e0 = 0; e0 < E; e0 += kWave) {
             const int e = e0 + lane;
-            const long long v = e < E ? (long long)lengths[e] : 0;
-            const long long inc = wave_inclusive_scan(v);
+            long long len = 0;
+            int32_t bef = 0;
+            if (e < E)
+                for (int w = 0; w < WPB; ++w) {
+                    len += s_tot[w * E + e];
+                    bef += s_bef[w * E + e];
+                }
+            const long long inc = wave_inclusive_scan(len);
             if (e < E) {
-                s_next[e] = (int32_t)(run + inc - v) + chunk_base[(int64_t)c * E + e];
-                if (c == 0) offsets[e] = run + inc - v;
+                s_base[e] = (int32_t)(run + inc - len) + bef;
+                if (c == 0) {
+                    lengths[e] = len;
+                    offsets[e] = run + inc - len;
+                }
             }
             run += wave_bcast(inc, kWave - 1);
         }
-        if (c == 0 && lane == 0) offsets[E] = run;
-        // positions dropped for an out-of-range expert id leave a tail behind the last expert's
-        // rows: it holds zeros rather than whatever the buffer held (normally the tail is empty)
-        if (c == 0)
+        if (c == 0) {
+            if (lane == 0) offsets[E] = run;
+            // positions dropped for an out-of-range expert id leave a tail behind the last expert's
+            // rows: it holds zeros rather than whatever the buffer held (normally the tail is empty)
             for (long long i = run + lane; i < (long long)num_tokens * K; i += kWave) {
                 gate_index[i] = 0;
                 token_index[i] = 0;
             }
+            if (bad_count) {
+                long long bad = 0;
+                if (bad_part)
+                    for (int cc = lane; cc < num_chunks; cc += kWave) bad += bad_part[cc];
+#pragma unroll
+                for (int o = 32; o >= 1; o >>= 1) bad += __shfl_xor(bad, o, kWave);
+                if (lane == 0) *bad_count = bad;
+            }
+        }
     }
     __syncthreads();
+    // phase 3: the counts of the earlier waves of the chunk (LDS) on top of the chunk's base
+    int32_t at[16];             // E <= 1024: at most 16 entries per lane
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int e = i * kWave + lane;
+        at[i] = 0;
+        if (e < E) {
+            at[i] = s_base[e];
+            for (int w = 0; w < wave; ++w) at[i] += s_next[w * E + e];
+        }
+    }
+    __syncthreads();            // every wave has read the counts before anyone overwrites them
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int e = i * kWave + lane;
+        if (e < E) s_next[wave * E + e] = at[i];
+    }
+    __syncthreads();
+    int32_t* next = s_next + wave * E;
     const int tpi = kWave / K;
-    const int64_t t_begin = (int64_t)c * tokens_per_chunk;
-    int64_t t_end = t_begin + tokens_per_chunk;
+    const int64_t t_begin = ((int64_t)c * WPB + wave) * tokens_per_wave;
+    int64_t t_end = t_begin + tokens_per_wave;
     if (t_end > num_tokens) t_end = num_tokens;
+    const int64_t passes = (tokens_per_wave + tpi - 1) / tpi;     // the same for every wave (barriers below)
     const int tok_in_iter = lane / K;
     const int slot = lane - tok_in_iter * K;
     const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    for (int64_t t0 = t_begin; t0 < t_end; t0 += tpi) {
-        const int64_t t = t0 + tok_in_iter;
+    for (int64_t pass = 0; pass < passes; ++pass) {
+        const int64_t t = t_begin + pass * tpi + tok_in_iter;
         const bool live = tok_in_iter < tpi && t < t_end;
         const int64_t p = t * K + slot;
         const uint32_t e = live ? compact[p] : (uint32_t)kBadExpert;
@@ -306,10 +460,10 @@ __global__ __launch_bounds__(kWave) void scatter_kernel(const uint16_t* __restri
         const int before = __popcll(same & lt_mask);
         const int count = __popcll(same);
         int32_t base = 0;
-        if (counted) base = s_next[e];
-        __syncthreads();
-        if (counted && before == 0) s_next[e] = base + count;
-        __syncthreads();
+        if (counted) base = next[e];
+        wave_lds_fence();
+        if (counted && before == 0) next[e] = base + count;
+        wave_lds_fence();
         const int64_t dst = (int64_t)base + before;
         // rank of this slot among the token's K slots, ordered by (expert, slot)
         int rank = 0;
@@ -333,39 +487,41 @@ int ceil_log2(int v) {
     return b;
 }
 
-int launch_sort(const uint16_t* compact, int32_t* chunk_hist, const RoutePlan& plan, int64_t T, int E,
-                int K, int64_t* lengths, int64_t* offsets, int64_t* gate_index, int64_t* token_index,
-                int64_t* reverse_index, hipStream_t stream) {
-    const int64_t total_pos = T * K;
-    hist_kernel<<<plan.num_chunks, kWave, E * sizeof(int32_t), stream>>>(
-        compact, total_pos, plan.tokens_per_chunk * K, E, chunk_hist);
-    scan_kernel<<<E, 256, 0, stream>>>(chunk_hist, plan.num_chunks, E, lengths);
-    scatter_kernel<<<plan.num_chunks, kWave, E * sizeof(int32_t), stream>>>(
-        compact, T, plan.tokens_per_chunk, E, K, ceil_log2(E), chunk_hist, lengths, offsets, gate_index,
-        token_index, reverse_index);
+int launch_sort(const RouteScratch& ws, const RoutePlan& plan, bool have_bad, int64_t T, int E, int K,
+                int64_t* lengths, int64_t* offsets, int64_t* gate_index, int64_t* token_index,
+                int64_t* reverse_index, int64_t* bad_count, hipStream_t stream) {
+    const size_t lds = (size_t)(3 * plan.wpb + 1) * E * sizeof(int32_t);
+    scan_scatter_kernel<<<plan.num_chunks, plan.wpb * kWave, lds, stream>>>(
+        ws.compact, T, plan.tokens_per_wave, E, K, ceil_log2(E), plan.num_chunks, ws.sub_hist, ws.tot_hist,
+        have_bad ? ws.bad_part : nullptr, lengths, offsets, gate_index, token_index, reverse_index, bad_count);
     return check_launch("routing sort");
 }
 
 template <typename T, int LPT, int VPL>
 void launch_topk(const void* scores, int64_t T_, int E, int K, int renorm, int64_t* topk_idx,
-                 void* gates, uint16_t* compact, hipStream_t stream) {
-    constexpr int tokens_per_block = (256 / kWave) * (kWave / LPT);
-    const int64_t blocks = (T_ + tokens_per_block - 1) / tokens_per_block;
-    topk_kernel<T, LPT, VPL><<<(unsigned)blocks, 256, 0, stream>>>(
-        (const T*)scores, T_, E, K, renorm, topk_idx, (T*)gates, compact);
+                 void* gates, const RouteScratch& ws, const RoutePlan& plan, hipStream_t stream) {
+    const size_t lds = (size_t)plan.wpb * E * sizeof(int32_t);
+    if (plan.wpb == 16)
+        topk_hist_kernel<T, LPT, VPL, 16><<<plan.num_chunks, 16 * kWave, lds, stream>>>(
+            (const T*)scores, T_, E, K, renorm, plan.tokens_per_wave, topk_idx, (T*)gates, ws.compact, ws.sub_hist,
+            ws.tot_hist);
+    else
+        topk_hist_kernel<T, LPT, VPL, 4><<<plan.num_chunks, 4 * kWave, lds, stream>>>(
+            (const T*)scores, T_, E, K, renorm, plan.tokens_per_wave, topk_idx, (T*)gates, ws.compact, ws.sub_hist,
+            ws.tot_hist);
 }
 
 template <typename T>
 int dispatch_topk(const void* scores, int64_t T_, int E, int K, int renorm, int64_t* topk_idx,
-                  void* gates, uint16_t* compact, hipStream_t stream) {
-#define FMOE_TOPK(LPT, VPL) launch_topk<T, LPT, VPL>(scores, T_, E, K, renorm, topk_idx, gates, compact, stream)
+                  void* gates, const RouteScratch& ws, const RoutePlan& plan, hipStream_t stream) {
+#define FMOE_TOPK(LPT, VPL) launch_topk<T, LPT, VPL>(scores, T_, E, K, renorm, topk_idx, gates, ws, plan, stream)
     if (E <= 8) FMOE_TOPK(8, 1);
     else if (E <= 16) FMOE_TOPK(16, 1);
-    else if (E <= 32) FMOE_TOPK(32, 1);
-    else if (E <= 64) FMOE_TOPK(64, 1);
-    else if (E <= 128) FMOE_TOPK(64, 2);
-    else if (E <= 256) FMOE_TOPK(64, 4);
-    else if (E <= 512) FMOE_TOPK(64, 8);
+    else if (E <= 32) FMOE_TOPK(16, 2);
+    else if (E <= 64) FMOE_TOPK(16, 4);
+    else if (E <= 128) FMOE_TOPK(16, 8);
+    else if (E <= 256) FMOE_TOPK(16, 16);
+    else if (E <= 512) FMOE_TOPK(16, 32);
     else return fail(FMOE_ERR_UNSUPPORTED, "fmoe_route_topk: E=%d > 512", E);
 #undef FMOE_TOPK
     return FMOE_OK;
@@ -387,9 +543,10 @@ int check_common(int64_t T, int E, int K, const void* workspace, size_t ws_bytes
     return FMOE_OK;
 }
 
-__global__ void empty_routing_kernel(int E, int64_t* lengths, int64_t* offsets) {
+__global__ void empty_routing_kernel(int E, int64_t* lengths, int64_t* offsets, int64_t* bad_count) {
     for (int e = threadIdx.x; e < E; e += blockDim.x) lengths[e] = 0;
     for (int e = threadIdx.x; e <= E; e += blockDim.x) offsets[e] = 0;
+    if (bad_count && threadIdx.x == 0) *bad_count = 0;
 }
 
 }  // namespace
@@ -412,20 +569,19 @@ static int route_topk_impl(const char* who, const void* scores, int score_dtype,
     FMOE_REQUIRE(score_dtype == FMOE_F32 || score_dtype == FMOE_BF16, "%s: scores must be fp32 or bf16", who);
     FMOE_REQUIRE(lengths && offsets, "%s: lengths/offsets are NULL", who);
     if (T == 0) {
-        empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets);
+        empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets, nullptr);
         return check_launch(who);
     }
     FMOE_REQUIRE(scores && topk_idx && gates && gate_index && token_index && reverse_index,
                  "%s: NULL tensor pointer", who);
     const RoutePlan plan = make_plan(T, E, K);
-    uint16_t* compact = (uint16_t*)workspace;
-    int32_t* chunk_hist = (int32_t*)((char*)workspace + plan.compact_bytes);
+    const RouteScratch ws = carve(workspace, plan);
     int rc = score_dtype == FMOE_F32
-                 ? dispatch_topk<float>(scores, T, E, K, renorm, topk_idx, gates, compact, stream)
-                 : dispatch_topk<uint16_t>(scores, T, E, K, renorm, topk_idx, gates, compact, stream);
+                 ? dispatch_topk<float>(scores, T, E, K, renorm, topk_idx, gates, ws, plan, stream)
+                 : dispatch_topk<uint16_t>(scores, T, E, K, renorm, topk_idx, gates, ws, plan, stream);
     if (rc) return rc;
-    return launch_sort(compact, chunk_hist, plan, T, E, K, lengths, offsets, gate_index, token_index,
-                       reverse_index, stream);
+    return launch_sort(ws, plan, false, T, E, K, lengths, offsets, gate_index, token_index, reverse_index, nullptr,
+                       stream);
 }
 
 extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K, int renorm,
@@ -443,8 +599,9 @@ extern "C" int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, i
 // until the process ends.  In host code `scratch` is only a handle for hipGetSymbolAddress;
 // the address kernels and copies use is the per-device pointer looked up below.
 static constexpr size_t kStaticCompactBytes = (size_t)FMOE_ROUTE_STATIC_MAX_POSITIONS * sizeof(uint16_t);
-static constexpr size_t kStaticHistBytes = (size_t)kMaxChunks * FMOE_ROUTE_STATIC_MAX_EXPERTS * sizeof(int32_t);
-static constexpr size_t kStaticScratchBytes = kStaticCompactBytes + kStaticHistBytes + 512;
+// (16 waves per block up to 256 experts, 4 beyond: 17 * 256 > 5 * 512)
+static constexpr size_t kStaticHistBytes = (size_t)kMaxChunks * (kMaxRouteWaves + 1) * 256 * sizeof(int32_t);
+static constexpr size_t kStaticScratchBytes = kStaticCompactBytes + kStaticHistBytes + kMaxChunks * 4 + 1280;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 static constexpr int kMaxDevices = 64;
@@ -498,18 +655,16 @@ extern "C" int fmoe_route_from_topk(const int64_t* topk_idx, int64_t T, int E, i
     hipStream_t stream = (hipStream_t)stream_;
     if (int rc = check_common(T, E, K, workspace, workspace_bytes, "fmoe_route_from_topk")) return rc;
     FMOE_REQUIRE(lengths && offsets, "fmoe_route_from_topk: lengths/offsets are NULL");
-    if (bad_count) zero_i64_kernel<<<1, 1, 0, stream>>>(bad_count);
     if (T == 0) {
-        empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets);
+        empty_routing_kernel<<<1, 256, 0, stream>>>(E, lengths, offsets, bad_count);
         return check_launch("fmoe_route_from_topk");
     }
     FMOE_REQUIRE(topk_idx && gate_index && token_index && reverse_index,
                  "fmoe_route_from_topk: NULL tensor pointer");
     const RoutePlan plan = make_plan(T, E, K);
-    uint16_t* compact = (uint16_t*)workspace;
-    int32_t* chunk_hist = (int32_t*)((char*)workspace + plan.compact_bytes);
-    const int64_t n = T * K;
-    compact_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(topk_idx, n, E, compact, bad_count);
-    return launch_sort(compact, chunk_hist, plan, T, E, K, lengths, offsets, gate_index, token_index,
-                       reverse_index, stream);
+    const RouteScratch ws = carve(workspace, plan);
+    compact_hist_kernel<<<plan.num_chunks, plan.wpb * kWave, ((size_t)plan.wpb * E + plan.wpb) * sizeof(int32_t), stream>>>(
+        topk_idx, T, E, K, plan.tokens_per_wave, ws.compact, ws.sub_hist, ws.tot_hist, ws.bad_part);
+    return launch_sort(ws, plan, true, T, E, K, lengths, offsets, gate_index, token_index, reverse_index, bad_count,
+                       stream);
 }

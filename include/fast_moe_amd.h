@@ -94,7 +94,7 @@ int fmoe_route_topk(const void* scores, int score_dtype, int64_t T, int E, int K
 
 /*
  * fmoe_route_topk without a workspace argument and without any allocation: the scratch lives in
- * device memory that is part of the library image (3 MiB per GPU the library runs on, held until
+ * device memory that is part of the library image (6.3 MiB per GPU the library runs on, held until
  * the process ends).  No counterpart in the reference.  For callers that cannot allocate: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments
  * and results as fmoe_route_topk, bit for bit.
