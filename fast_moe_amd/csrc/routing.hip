@@ -5,10 +5,12 @@
 // reproducible bit for bit.
 //
 // Two launches on one stream, no host synchronisation.  The tokens are cut into up to 256
-// chunks (one block of 4 waves each, a wave owns a contiguous quarter of its chunk):
-//   1. topk_hist_kernel (or compact_hist_kernel for caller-supplied ids): selection by rank
-//      counting, one token per LPT lanes; every wave counts the experts of its tokens in LDS ->
-//      sub_hist[chunk][wave][e], tot_hist[chunk][e]
+// chunks (one block each: 16 waves up to 256 experts, 4 beyond; a wave owns a contiguous
+// share of its chunk):
+//   1. topk_hist_kernel (or compact_hist_kernel for caller-supplied ids): a token's scores sit
+//      in a group of 8 or 16 lanes (4 to 8 tokens per wave); K rounds of a group argmax on the
+//      DPP network select in descending order, ties to the lower expert id; every wave counts
+//      the experts of its tokens in LDS -> sub_hist[chunk][wave][e], tot_hist[chunk][e]
 //   2. scan_scatter_kernel: every block sums tot_hist over the chunks before it (and over all
 //      chunks: lengths; wave scan over the experts: offsets), every wave adds the counts of
 //      the waves before it in its chunk and then places its positions: a wave-level
