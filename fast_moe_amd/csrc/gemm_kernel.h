@@ -288,8 +288,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     auto run = [&](auto has_bias_c, auto has_aux_c) {
         constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
         constexpr bool HAS_AUX = SWIGLU && decltype(has_aux_c)::value;   // keep the pre-activations (training)
-        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && !FP8 && FN_OUT == 2;   // (the e4m3 kernels have no registers to spare for it)
-        constexpr bool PAIRS = FP8 && !SWIGLU;      // the cheap half of it, per 16-column group (measured: no gain on the SwiGLU epilogues)
+        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && FN_OUT == 2;   // plain and SiLU epilogues of the ring kernel, bf16 and e4m3
         // per-column biases of this lane, indexed like rsw
         float bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
         // with a bias, at least one of the two pointers is set: both loads go through a valid
@@ -483,32 +482,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         }
                     // base: first element of the 32-row block's first row (wave-uniform)
                     auto store = [&](const float (&val)[2][4], uint16_t* base, int64_t stride) {
-                        if constexpr (ALWAYS_VEC && PAIRS) {
-                            // Adjacent lanes first trade one 8-byte piece (the even lane of a pair
-                            // keeps columns nq..nq+7 of both rows' lane halves, the odd one
-                            // nq+8..nq+15), then the halves of the wave trade as below, by row:
-                            // lanes 2m, 2m+1 end up with row 2m's 32 contiguous bytes, lanes
-                            // 2m+32, 2m+33 with row 2m+1's (the store unit merges adjacent lanes only).
-                            int l = lane;
-                            asm volatile("" : "+v"(l));
-                            const bool odd = (l & 1) != 0;
-                            uint32_t a[2], b[2];
-#pragma unroll
-                            for (int d = 0; d < 2; ++d) {
-                                const uint32_t p0 = pack_bf16(val[0][2 * d], val[0][2 * d + 1]);
-                                const uint32_t p1 = pack_bf16(val[1][2 * d], val[1][2 * d + 1]);
-                                const uint32_t send = odd ? p0 : p1;
-                                const uint32_t recv = (uint32_t)__builtin_amdgcn_mov_dpp((int)send, 0xB1, 0xF, 0xF, true);
-                                const u32x2 t = __builtin_amdgcn_permlane32_swap(odd ? recv : p0, odd ? p1 : recv, false, false);
-                                a[d] = t[0];
-                                b[d] = t[1];
-                            }
-                            const int row = 2 * ((l & 31) >> 1) + (l >> 5);
-                            const uint32_t lane_off = ((uint32_t)row * (uint32_t)stride + (uint32_t)(8 * (l & 1))) * 2u;
-                            if (wm * TM + fm * 32 + row < rows_valid && nq + 8 * (l & 1) + 7 < p.N)
-                                *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(base + nq) + lane_off) =
-                                    u32x4{a[0], a[1], b[0], b[1]};
-                        } else if (ALWAYS_VEC || p.vec_store) {
+                        if (ALWAYS_VEC || p.vec_store) {
                             const uint32_t lane_off = lane_offset(stride);
                             // pair the quads of the two lane halves: low lanes end up with columns
                             // nq..nq+7, high lanes with nq+8..nq+15 of their row
