@@ -1792,12 +1792,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             auto tile_steps = [&](auto half_c) {
                 const int tile_kt = KWIN ? cur.kt : KT;
-                // The first double step stands outside the loop, and every wave runs it in the
-                // second half's form (issue after A', vmcnt(0) before it): that explicit wait,
-                // which finds nothing young in flight, also settles whatever the compiler still
-                // counts as pending from the tile's set-up or the last epilogue (spill reloads,
-                // the row-index loads).  Left pending, their waits land inside the loop, where
-                // each one drains the LDS-DMA stream the compiler cannot see, every iteration.
+                // (whatever the compiler still counts as pending from the tile's set-up or the last
+                // epilogue, spill reloads and the row-index loads, is settled by the counted wait at
+                // the epilogue's end: left pending, such a wait lands inside this loop, where it
+                // drains the LDS-DMA stream, which the compiler cannot see, on every iteration)
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) {
                     double_step(half_c, std::false_type{});
 #ifdef FMOE_TRACE
