@@ -148,6 +148,19 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
+// 16-byte store through a buffer descriptor over [base, base + 2 GiB): a lane whose offset is
+// kDropLane lies outside the descriptor's range and the hardware drops its part, so the
+// instruction is issued whatever the lanes' predicates are.  The compiler then knows how many
+// stores follow an older load and waits for that load with an exact count; behind stores it
+// may or may not have branched around it has to wait for everything in flight, the LDS-DMA
+// stream and the stores' own round trip included.  base is wave-uniform (scalar registers).
+constexpr uint32_t kDropLane = 0x80000000u;
+__device__ __forceinline__ void store16_uniform_base(const void* base, uint32_t lane_offset, u32x4 v) {
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)kDropLane, 0x00020000);
+    __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)lane_offset, 0, 0);
+}
+
 // ------------------------------------------------------------------------ epilogue
 // acc[fn][fm][v]: fragment (fn, fm) of the wave tile, v = 4*g + j <-> output row
 // (lane & 31) of fragment row block fm, output column 32*fn + 8*g + 4*(lane >> 5) + j.
@@ -159,11 +172,20 @@ __device__ __forceinline__ void wait_vmcnt() {   // s_waitcnt vmcnt(N) only
 // condition), so row numbers and row_index values fit 32 bits.
 // OUT2: an expert's output rows are split in two halves that go to two tensors (p.out2; the
 // weight gradients of two matrices from one GEMM); a 32-row block lies in one half.
+// after_stores(): called at the very end, in the same straight-line code as the stores and the
+// counted wait behind them, where the compiler's own count of what is still in flight is exact
+// (behind the join of the epilogue's variants it is not: it has to assume the path that stored
+// nothing).  The ring kernel converts the row indices it fetched before the epilogue there.
+struct NoAfterStores {
+    __device__ __forceinline__ void operator()() const {}
+};
+
 template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false, bool ROWS32 = false,
-          bool OUT2 = false>
+          bool OUT2 = false, typename AfterStores = NoAfterStores>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
-                                              int lane, uint64_t* ets = nullptr) {
+                                              int lane, AfterStores after_stores = AfterStores(),
+                                              uint64_t* ets = nullptr) {
     constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
     constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
     const int khalf = lane >> 5;
@@ -407,9 +429,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     uint16_t* base = obase + i * p.out_stride + col0;
-                    if (wm * TM + fm * 32 + quad_row + i < rows_valid && col + 7 < p.N)
-                        *reinterpret_cast<u32x4*>(reinterpret_cast<uint8_t*>(base) + lane_off) =
-                            u32x4{ch[i][0], ch[i][1], ch[i][2], ch[i][3]};
+                    const bool ok = wm * TM + fm * 32 + quad_row + i < rows_valid && col + 7 < p.N;
+                    store16_uniform_base(base, ok ? lane_off : kDropLane, u32x4{ch[i][0], ch[i][1], ch[i][2], ch[i][3]});
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 continue;
@@ -482,7 +503,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         }
                     // base: first element of the 32-row block's first row (wave-uniform)
                     auto store = [&](const float (&val)[2][4], uint16_t* base, int64_t stride) {
-                        if (ALWAYS_VEC || p.vec_store) {
+                        if constexpr (ALWAYS_VEC) {
+                            const uint32_t lane_off = lane_offset(stride);
+                            const u32x2 s0 = __builtin_amdgcn_permlane32_swap(pack_bf16(val[0][0], val[0][1]),
+                                                                              pack_bf16(val[1][0], val[1][1]), false, false);
+                            const u32x2 s1 = __builtin_amdgcn_permlane32_swap(pack_bf16(val[0][2], val[0][3]),
+                                                                              pack_bf16(val[1][2], val[1][3]), false, false);
+                            const int nb = nq + 8 * khalf;
+                            const bool ok = row_ok[fm] && nb + 7 < p.N;
+                            store16_uniform_base(base + nq, ok ? lane_off : kDropLane, u32x4{s0[0], s1[0], s0[1], s1[1]});
+                        } else if (p.vec_store) {
                             const uint32_t lane_off = lane_offset(stride);
                             // pair the quads of the two lane halves: low lanes end up with columns
                             // nq..nq+7, high lanes with nq+8..nq+15 of their row
@@ -538,6 +568,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         // which the compiler cannot see, on every iteration.
         FMOE_EPI_STAMP(FM);
         wait_vmcnt<FM * FN_OUT * 2 * (HAS_AUX ? 3 : 1)>();      // (the scalar-store path issues more)
+        after_stores();
     };
     if (SWIGLU && p.aux) {
         if (p.bias || p.bias2) run(std::true_type{}, std::true_type{});
@@ -1412,14 +1443,12 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     int ikt = 0;                            // next K-slice to issue inside the issue tile
     int issued = 0;                         // items issued so far
     int islot = 0;                          // issued % STAGES
-    // EARLY_ROWS: the row indices of a tile are fetched two tiles ahead, before the epilogue of
-    // the tile in between, and turned into offsets at the start of the tile before theirs: by
-    // then they have long arrived, and no load the compiler knows of is in flight while the
-    // main loop runs (its wait for one would also drain the LDS-DMA stream, which it cannot
-    // see).  Otherwise they are fetched at the start of the tile before theirs and converted
-    // when the issue side gets there: two registers fewer across the main loop, which is what
-    // the e4m3 kernels, at the limit of the register file, need more.
-    constexpr bool EARLY_ROWS = !FP8;
+    // The row indices of a tile are fetched two tiles ahead, before the epilogue of the tile in
+    // between, and turned into offsets right behind that epilogue: by then they have long
+    // arrived, the wait the compiler needs for them counts the epilogue's stores exactly (they
+    // are issued unconditionally, see store16_uniform_base), and no load the compiler knows of
+    // is in flight while the main loop runs (its wait for one would also drain the LDS-DMA
+    // stream, which it cannot see).
     int64_t ridx_next[XI];
     uint32_t xoff_next[XI];
 #pragma unroll
@@ -1435,7 +1464,6 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         make_ptrs(cur, x0);
     }
     auto enter_next = [&]() {               // the issue side moves on to the next tile
-        if (!EARLY_ROWS) rows_to_offsets(ridx_next, xoff_next);
         make_ptrs(nxt, xoff_next);
     };
     auto issue_next = [&]() {
@@ -1478,6 +1506,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         }
     };
     prefetch_next();
+    rows_to_offsets(ridx_next, xoff_next);
     if (PAIR) {
         issue_next();                       // items 0..3
         issue_next();
@@ -1506,8 +1535,6 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         FMOE_TRACE_STAMP(0);
         if (p.trace) tstamp[4] = __builtin_amdgcn_s_memtime();
 #endif
-        if (EARLY_ROWS) rows_to_offsets(ridx_next, xoff_next);      // the tile after this one
-        else if (tile_i > 0) prefetch_next();
 
         auto mma_slice = [&]() {
             const uint8_t* sx = smem + cslot * TL::STAGE_BYTES;
@@ -1635,7 +1662,13 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             // sched_barrier(0) pins the order "reads of the next block, then the MFMAs of this
             // one"; left alone the scheduler sinks the reads to just before their first use.
             int kitem = 0;                  // number, inside the tile, of the item in slot cslot
-            auto double_step = [&](auto half_c, auto last_c, auto mask_c) {
+            // skip_wait (wave-uniform): the pair this step would wait for is known to have landed.  That
+            // holds for the first step of every tile but the block's first: the pair was issued before
+            // the previous epilogue, whose stores are all issued whatever their lanes' predicates
+            // (store16_uniform_base) and followed by a wait that leaves at most that many operations
+            // in flight, i.e. nothing older than the stores.  The counted wait here would sit out the
+            // stores' own round trip instead (one counter serves loads and stores, in order).
+            auto double_step = [&](auto half_c, auto last_c, auto mask_c, bool skip_wait) __attribute__((always_inline)) {
                 constexpr int HALF = decltype(half_c)::value;
                 constexpr bool LAST = decltype(last_c)::value;   // last of the tile: no fragments kept over the epilogue
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
@@ -1674,8 +1707,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 if constexpr (HALF != 0) interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 // pair (c+2, c+3) is older than the 2L instructions the first half just issued
-                if (HALF == 0) wait_vmcnt<2 * L>();
-                else wait_vmcnt<0>();
+                if (!skip_wait) {
+                    if (HALF == 0) wait_vmcnt<2 * L>();
+                    else wait_vmcnt<0>();
+                }
                 barrier();                  // A'
                 if (!LAST) load_block(wfa, xfa, s2, 0, kitem + 2, mask_c);
                 if constexpr (HALF == 1 || LAST) __builtin_amdgcn_sched_barrier(0);
@@ -1687,10 +1722,12 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             // the issue side runs 4 items ahead: it enters the next tile 4 items before the end;
             // the last two double steps hold the end of an XTR tile's window and mask it
-            auto tile_steps = [&](auto half_c) {
+            auto tile_steps = [&](auto half_c) __attribute__((always_inline)) {
                 const int tile_kt = KWIN ? cur.kt : KT;
+                bool landed = tile_i > 0;       // the first step's pair landed before the previous epilogue's stores
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) {
-                    double_step(half_c, std::false_type{}, std::false_type{});
+                    double_step(half_c, std::false_type{}, std::false_type{}, landed);
+                    landed = false;
 #ifdef FMOE_TRACE
                     if (kt < 8) FMOE_TRACE_STAMP(6 + kt / 2);
 #endif
@@ -1698,9 +1735,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 FMOE_TRACE_STAMP(10);
                 enter_next();
                 ikt = 0;
-                double_step(half_c, std::false_type{}, std::true_type{});
+                double_step(half_c, std::false_type{}, std::true_type{}, landed);
                 FMOE_TRACE_STAMP(11);
-                double_step(half_c, std::true_type{}, std::true_type{});
+                double_step(half_c, std::true_type{}, std::true_type{}, false);
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
                 wait_vmcnt<2 * L>();
@@ -1756,7 +1793,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             };
-            auto double_step = [&](auto half_c, auto last_c) {
+            auto double_step = [&](auto half_c, auto last_c, bool skip_wait) __attribute__((always_inline)) {   // skip_wait: as in the bf16 loop
                 constexpr int HALF = decltype(half_c)::value;
                 constexpr bool LAST = decltype(last_c)::value;
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
@@ -1781,8 +1818,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 __builtin_amdgcn_sched_barrier(0);
                 mma_block(qwb, qx0, 0, std::integral_constant<bool, HALF == 0>{});
                 __builtin_amdgcn_sched_barrier(0);
-                if (HALF == 0) wait_vmcnt<2 * L>();
-                else wait_vmcnt<0>();
+                if (!skip_wait) {
+                    if (HALF == 0) wait_vmcnt<2 * L>();
+                    else wait_vmcnt<0>();
+                }
                 barrier();                  // A'
                 if (!LAST) load_w_x0(qwa, qx0, s2);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1790,14 +1829,16 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 __builtin_amdgcn_sched_barrier(0);
                 cslot = s2;
             };
-            auto tile_steps = [&](auto half_c) {
+            auto tile_steps = [&](auto half_c) __attribute__((always_inline)) {
                 const int tile_kt = KWIN ? cur.kt : KT;
                 // (whatever the compiler still counts as pending from the tile's set-up or the last
                 // epilogue, spill reloads and the row-index loads, is settled by the counted wait at
                 // the epilogue's end: left pending, such a wait lands inside this loop, where it
                 // drains the LDS-DMA stream, which the compiler cannot see, on every iteration)
+                bool landed = tile_i > 0;
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) {
-                    double_step(half_c, std::false_type{});
+                    double_step(half_c, std::false_type{}, landed);
+                    landed = false;
 #ifdef FMOE_TRACE
                     if (kt < 8) FMOE_TRACE_STAMP(6 + kt / 2);
 #endif
@@ -1805,9 +1846,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 FMOE_TRACE_STAMP(10);
                 enter_next();
                 ikt = 0;
-                double_step(half_c, std::false_type{});
+                double_step(half_c, std::false_type{}, landed);
                 FMOE_TRACE_STAMP(11);
-                double_step(half_c, std::true_type{});
+                double_step(half_c, std::true_type{}, false);
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
                 wait_vmcnt<2 * L>();
@@ -1839,16 +1880,19 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         FMOE_TRACE_STAMP(1);
         const TileInfo done = cur;
         cur = nxt;          // valid when another tile follows
-        if (EARLY_ROWS) prefetch_next();    // nxt: the tile after that one; its row indices arrive during the epilogue
+        prefetch_next();    // nxt: the tile after that one; its row indices arrive during the epilogue
         FMOE_TRACE_STAMP(2);
 
+        auto convert_rows = [&]() __attribute__((always_inline)) {
+            rows_to_offsets(ridx_next, xoff_next);  // of the tile after the next one
+        };
 #ifdef FMOE_TRACE
         gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(
-            p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane,
+            p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane, convert_rows,
             (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2)) ? tstamp + 12 : nullptr);
 #else
         gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
-                                                                done.rows_valid, wm, wn, lane);
+                                                                done.rows_valid, wm, wn, lane, convert_rows);
 #endif
 #ifdef FMOE_TRACE
         FMOE_TRACE_STAMP(3);
