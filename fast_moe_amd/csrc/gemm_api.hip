@@ -96,6 +96,7 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     p.index_shift = -1;
     for (int s = 0; s < 31; ++s)
         if (d->index_div == (1 << s)) p.index_shift = s;
+    magic_u31(d->index_div, &p.index_magic, &p.index_magic_shift);     // (read when index_div is no power of two)
     p.total_rows = d->total_rows;
     p.a_rows = d->a_rows;
     p.a = (const uint8_t*)d->a;

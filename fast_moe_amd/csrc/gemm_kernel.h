@@ -48,6 +48,13 @@ struct GemmParams {
     const int64_t* row_index;
     int E, N, K, index_div;
     int index_shift;                    // log2(index_div) when it is a power of two, else -1
+    // otherwise, for 0 <= v < 2^31: v / index_div == mulhi(v, index_magic) >> index_magic_shift
+    // (magic = ceil(2^p / d), p = 31 + ceil(log2 d): the error of the product stays below 2^p)
+    uint32_t index_magic;
+    int index_magic_shift;
+    // the same for the tile scheduler of the paired ring: v / (kGroupM * n_tiles) for v < 2^31
+    uint32_t group_magic;
+    int group_magic_shift;
     int64_t total_rows, a_rows;
     const uint8_t* a;
     int64_t a_stride_row, a_stride_e;   // elements
@@ -100,6 +107,35 @@ constexpr int kNumXcd = 8;
 
 __device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) {
     return v < lo ? lo : (v > hi ? hi : v);
+}
+
+// two consecutive int64 from a wave-uniform address through the scalar cache (read only)
+__device__ __forceinline__ void scalar_load_i64x2(const int64_t* ptr, int64_t& a, int64_t& b) {
+    typedef __attribute__((ext_vector_type(4))) int i32x4;
+    i32x4 v;
+    asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(ptr) : "memory");
+    a = (int64_t)(((uint64_t)(uint32_t)v[1] << 32) | (uint32_t)v[0]);
+    b = (int64_t)(((uint64_t)(uint32_t)v[3] << 32) | (uint32_t)v[2]);
+}
+
+// row_index value -> source row, for values below 2^31 (the paired ring: total_rows < 2^31): a
+// shift or one multiply by wave-uniform constants, no division sequence and nothing per lane for
+// the compiler to keep across the tile loop.  Negative (malformed) values give some row; the
+// callers clamp.
+__device__ __forceinline__ int32_t div_index32(const GemmParams& p, int32_t v) {
+    if (p.index_shift >= 0) return v >> p.index_shift;
+    return (int32_t)(__umulhi((uint32_t)v, p.index_magic) >> p.index_magic_shift);
+}
+
+// magic and shift with v / d == mulhi(v, magic) >> shift for every 0 <= v < 2^31 (d >= 3, or any
+// d >= 2 that is no power of two; powers of two from 4 on work as well)
+inline void magic_u31(int64_t d, uint32_t* magic, int* shift) {
+    int cl = 0;                             // ceil(log2 d)
+    while (((int64_t)1 << cl) < d) ++cl;
+    const int pw = 31 + cl;
+    const unsigned __int128 one = 1;
+    *magic = (uint32_t)((((one << pw) + (unsigned __int128)d - 1) / (unsigned __int128)d) & 0xffffffffu);
+    *shift = pw - 32;
 }
 
 __device__ __forceinline__ int64_t source_row(const GemmParams& p, int64_t r) {
@@ -188,6 +224,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                               uint64_t* ets = nullptr) {
     constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
     constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
+    // (ring kernel: everything derived from the lane number below is recomputed per tile; as
+    // tile-loop invariants the compiler keeps such values in registers across the main loop, or
+    // spills them and reloads them here behind a wait that drains the LDS-DMA stream)
+    if (ALWAYS_VEC) asm volatile("" : "+v"(lane));
     const int khalf = lane >> 5;
     const int64_t bias_row = (int64_t)expert * p.bias_se;
 #ifdef FMOE_TRACE
@@ -238,7 +278,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
             }
 #pragma unroll
             for (int fm = 0; fm < FM; ++fm)
-                src[fm] = p.index_shift >= 0 ? (src[fm] >> p.index_shift) : src[fm] / (row_t)p.index_div;
+                if (ROWS32) src[fm] = (row_t)div_index32(p, (int32_t)src[fm]);
+                else src[fm] = p.index_shift >= 0 ? (src[fm] >> p.index_shift) : src[fm] / (row_t)p.index_div;
         }
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
@@ -1070,7 +1111,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     const int64_t R = p.total_rows;
     int total_m;
     // register tables: lane l of entry i describes expert 64 * i + l
-    int r_first[NR], r_lo[NR], r_len[NR];     // first row tile, first row, rows
+    int r_end[NR];                            // row tiles up to and including this position
     // KWIN: the tables are in order of decreasing contraction window (the cost of an expert's
     // tiles), r_exp tells which expert sits at a position: dealing groups of tiles to the XCDs
     // back and forth then balances them whatever order the experts' loads come in.
@@ -1138,9 +1179,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             const int64_t lo = e_lo[i], len = e_len[i];
             const int tiles = (int)((len + BM - 1) / BM);
             const int inc = wave_inclusive_scan(tiles);
-            r_first[i] = run + inc - tiles;
-            r_lo[i] = (int)lo;
-            r_len[i] = (int)len;
+            r_end[i] = run + inc;
             run += uniform_lane(inc, kWave - 1);
         }
         total_m = run;
@@ -1165,7 +1204,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         }
         __syncthreads();
         total_m = s_tab[p.E];
-        r_first[0] = r_lo[0] = r_len[0] = 0;
+        r_end[0] = 0;
     }
     // The tiles of an XCD, numbered 0 .. xcd_count-1.  Without a contraction window: one
     // contiguous range of the tile order (neighbouring tiles share operands in the XCD's L2).
@@ -1196,41 +1235,65 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         xcd_begin = xcd * per_xcd;
         xcd_count = total_tiles - xcd_begin < per_xcd ? total_tiles - xcd_begin : per_xcd;
     }
+    // tile numbers of the paired ring fit 31 bits (the launcher checks): divisions by the group
+    // span are one scalar multiply by a constant the host prepared, no division sequence whose
+    // per-lane pieces the compiler would keep (or spill) across the tile loop
+    auto div_span = [&](int64_t v) -> int64_t {
+        if constexpr (PAIR) return (int64_t)(__umulhi((uint32_t)v, p.group_magic) >> p.group_magic_shift);
+        else return v / group_span;
+    };
     auto to_logical = [&](int64_t j) -> int64_t {
         if (!windowed) return xcd_begin + j;
-        const int64_t round = j / group_span;
+        const int64_t round = div_span(j);
         const int pos = (round & 1) ? kNumXcd - 1 - xcd : xcd;
-        return (round * kNumXcd + pos) * group_span + j % group_span;
+        return (round * kNumXcd + pos) * group_span + (j - round * group_span);
     };
 
     const int KT = p.K / BK;
     struct TileInfo { int expert; int nt; int64_t row0; int rows_valid; int64_t k_begin; int kt; int m0; int klen; };
     auto locate = [&](int64_t logical) -> TileInfo {
-        const int64_t group = logical / group_span;
+        const int64_t group = div_span(logical);
         const int first_m = (int)(group * kGroupM);
         const int gsize = total_m - first_m < kGroupM ? total_m - first_m : kGroupM;
         const int within = (int)(logical - group * group_span);
-        const int mt = first_m + within % gsize;
+        static_assert(kGroupM == 4, "the quotient below knows the group sizes 1..4");
+        const uint32_t uw = (uint32_t)within;
+        const int q = gsize == 4 ? (int)(uw >> 2)
+                      : gsize == 2 ? (int)(uw >> 1)
+                                   : gsize == 3 ? (int)(((uint64_t)uw * 0xAAAAAAABull) >> 33) : within;
+        const int mt = first_m + (within - q * gsize);
         TileInfo t;
-        t.nt = within / gsize;
+        t.nt = q;
         if constexpr (PAIR) {
-            // the tile's expert = number of experts whose row tiles all precede mt
+            // the tile's position = number of positions whose row tiles all precede mt; its first
+            // tile is where the position before it ends.  Only the running tile count is kept per
+            // position (one register per 64 experts); the expert's first row and row count come from
+            // offsets[] through the scalar cache: two loads that wait on their own counter, where a
+            // table register spilled to scratch is reloaded behind a wait that drains the LDS-DMA
+            // stream.  (Lane rl of every table register first, then a scalar select among them:
+            // selecting the register first reads as indexing an array by a run-time value, and the
+            // compiler then keeps the table in scratch memory.)
             int cnt = 0;
 #pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                const int e = i * kWave + lane;
-                const bool before = e < p.E && r_first[i] + (r_len[i] + BM - 1) / BM <= mt;
-                cnt += __builtin_popcountll(__ballot(before));
-            }
+            for (int i = 0; i < NR; ++i) cnt += __builtin_popcountll(__ballot(r_end[i] <= mt));
             cnt = __builtin_amdgcn_readfirstlane(cnt);
-            const int ri = cnt >> 6, rl = cnt & 63;
-            int vf = r_first[0], vl = r_lo[0], vn = r_len[0], ve = r_exp[0];
+            cnt = cnt < p.E ? cnt : p.E - 1;        // (unreachable for consistent offsets)
+            const int ri = cnt >> 6, rl = cnt & 63, pri = (cnt - 1) >> 6, prl = (cnt - 1) & 63;
+            int first = 0, ex = 0;
 #pragma unroll
-            for (int i = 1; i < NR; ++i)
-                if (ri == i) { vf = r_first[i]; vl = r_lo[i]; vn = r_len[i]; ve = r_exp[i]; }
-            const int first = uniform_lane(vf, rl), lo = uniform_lane(vl, rl), len = uniform_lane(vn, rl);
+            for (int i = 0; i < NR; ++i) {
+                const int f = uniform_lane(r_end[i], prl), x = KWIN ? uniform_lane(r_exp[i], rl) : 0;
+                if (cnt > 0 && pri == i) first = f;
+                if (ri == i) ex = x;
+            }
+            const int expert = KWIN ? ex : cnt;
+            int64_t o_lo, o_hi;
+            scalar_load_i64x2(p.offsets + expert, o_lo, o_hi);
+            o_lo = clamp_i64(o_lo, 0, R);
+            o_hi = clamp_i64(o_hi, 0, R);
+            const int lo = (int)o_lo, len = (int)(o_hi > o_lo ? o_hi - o_lo : 0);
             const int skip = (mt - first) * BM;
-            t.expert = KWIN ? uniform_lane(ve, rl) : cnt;
+            t.expert = expert;
             t.m0 = skip;
             t.row0 = (int64_t)lo + skip;
             const int left = len - skip;
@@ -1313,7 +1376,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
             int64_t s = ridx[i];
-            if (p.row_index) s = p.index_shift >= 0 ? (s >> p.index_shift) : s / p.index_div;
+            if (p.row_index) {
+                if (PAIR) s = div_index32(p, (int32_t)s);      // (values below 2^31, as in the epilogue)
+                else s = p.index_shift >= 0 ? (s >> p.index_shift) : s / p.index_div;
+            }
             s = clamp_i64(s, 0, p.a_rows - 1);
             out[i] = (uint32_t)(s * (p.a_stride_row * ESIZE)) + dma_swizzle(i);
         }
@@ -1963,6 +2029,11 @@ template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, b
 int launch_ring_cfg(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
+    if (TL::PAIR) {
+        if ((p.total_rows / TL::BM + p.E + kGroupM) * (int64_t)p.n_tiles >= ((int64_t)1 << 31))
+            return fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: more than 2^31 output tiles");
+        magic_u31((int64_t)kGroupM * p.n_tiles, &p.group_magic, &p.group_magic_shift);
+    }
     auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN, XTR>;
     static bool attr_done = false;
     if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
