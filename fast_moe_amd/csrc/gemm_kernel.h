@@ -208,6 +208,9 @@ __device__ __forceinline__ void store16_uniform_base(const void* base, uint32_t 
 // condition), so row numbers and row_index values fit 32 bits.
 // OUT2: an expert's output rows are split in two halves that go to two tensors (p.out2; the
 // weight gradients of two matrices from one GEMM); a 32-row block lies in one half.
+// ROW_IL: the two wave rows share the tile's 32-row blocks alternately (block 2*fm + wm belongs to
+// wave row wm) instead of owning one half of the tile each, so that a tile with few valid rows
+// leaves both with the same number of blocks to compute.
 // after_stores(): called at the very end, in the same straight-line code as the stores and the
 // counted wait behind them, where the compiler's own count of what is still in flight is exact
 // (behind the join of the epilogue's variants it is not: it has to assume the path that stored
@@ -217,7 +220,7 @@ struct NoAfterStores {
 };
 
 template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false, bool ROWS32 = false,
-          bool OUT2 = false, typename AfterStores = NoAfterStores>
+          bool OUT2 = false, bool ROW_IL = false, typename AfterStores = NoAfterStores>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
                                               int lane, AfterStores after_stores = AfterStores(),
@@ -251,11 +254,13 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         asm volatile("" : "+v"(l));
         return (uint32_t)(l & 31) * (uint32_t)stride * 2u + (uint32_t)(l >> 5) * 16u;
     };
+    // first tile row of the wave's row block fm
+    auto frag_row = [&](int fm) -> int { return ROW_IL ? (fm * 2 + wm) * 32 : wm * TM + fm * 32; };
     float rsa[FM];
     bool row_ok[FM];
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
-        row_ok[fm] = wm * TM + fm * 32 + (lane & 31) < rows_valid;
+        row_ok[fm] = frag_row(fm) + (lane & 31) < rows_valid;
         rsa[fm] = 1.0f;
     }
     // per-column reciprocal weight scales of this lane (e4m3): [fn][gp][q][j] <-> column
@@ -269,7 +274,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         row_t src[FM];
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm)
-            src[fm] = (row_t)(row0 + (row_ok[fm] ? wm * TM + fm * 32 + (lane & 31) : 0));
+            src[fm] = (row_t)(row0 + (row_ok[fm] ? frag_row(fm) + (lane & 31) : 0));
         if (p.row_index) {
 #pragma unroll
             for (int fm = 0; fm < FM; ++fm) {
@@ -452,7 +457,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                         ch[pr][d] = up ? recv : ch[pr][d];
                         ch[pr + 2][d] = up ? ch[pr + 2][d] : recv;
                     }
-                const int64_t block_row = row0 + wm * TM + fm * 32;
+                const int64_t block_row = row0 + frag_row(fm);
                 uint16_t* obase = p.out + block_row * p.out_stride;
                 if constexpr (OUT2) {
                     if (p.out2) {       // (as below: wave-uniform, forced into the two tensors)
@@ -470,7 +475,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     uint16_t* base = obase + i * p.out_stride + col0;
-                    const bool ok = wm * TM + fm * 32 + quad_row + i < rows_valid && col + 7 < p.N;
+                    const bool ok = frag_row(fm) + quad_row + i < rows_valid && col + 7 < p.N;
                     store16_uniform_base(base, ok ? lane_off : kDropLane, u32x4{ch[i][0], ch[i][1], ch[i][2], ch[i][3]});
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -576,7 +581,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                 }
                         }
                     };
-                    const int64_t block_row = row0 + wm * TM + fm * 32;
+                    const int64_t block_row = row0 + frag_row(fm);
                     uint16_t* obase = p.out + block_row * p.out_stride;
                     if constexpr (OUT2) {
                         if (p.out2) {       // (scalar arithmetic: everything here is wave-uniform)
@@ -1096,6 +1101,13 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;
     constexpr int XI = TL::XI, WI = TL::WI;
     constexpr int L = XI + WI;
+    // the two wave rows take the tile's 32-row blocks alternately (see slot_row_to_tile_row)
+    constexpr bool ROW_IL = !XTR && TL::WGM == 2 && FM == 4;
+    // SPARSE: a tile whose valid rows end in its first half (a short expert, or the rows an expert
+    // has beyond a multiple of the tile height) runs a second copy of the main loop that
+    // multiplies only the first two of every wave's four row blocks; the others hold no valid row.
+    constexpr bool SPARSE = ROW_IL && PAIR && !KWIN;
+    constexpr int ACT_SPARSE = FM / 2;
 
     extern __shared__ __align__(16) uint8_t smem[];
     int32_t* s_tab = reinterpret_cast<int32_t*>(smem + TL::TAB_OFF);   // [E+1] row-tile prefix
@@ -1355,12 +1367,20 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     };
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem;
 
+    // ROW_IL: row r of a ring slot's activation part (wave row r / TM reads it, as block
+    // (r % TM) / 32 of its four) holds the tile's row block 2 * block + wave row: the two wave rows
+    // take the tile's 32-row blocks alternately, and a tile with few valid rows leaves both the
+    // same number of blocks to multiply.
+    auto slot_row_to_tile_row = [&](int r) -> int {
+        if constexpr (!ROW_IL) return r;
+        else return (((r % TM) >> 5) * 2 + r / TM) * 32 + (r & 31);
+    };
     // source rows (row_index entries) of a tile, fetched ahead of the pointer computation
     auto fetch_rows = [&](const TileInfo& t, int64_t* ridx) {
         if constexpr (XTR) return;          // rows are not indexed: make_ptrs needs the tile only
 #pragma unroll
         for (int i = 0; i < XI; ++i) {
-            const int xr = dma_row(i);
+            const int xr = slot_row_to_tile_row(dma_row(i));
             const int64_t r = t.row0 + (xr < t.rows_valid ? xr : 0);
             ridx[i] = p.row_index ? p.row_index[r] : r;
         }
@@ -1672,8 +1692,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             // item: the slice's number inside the tile; mask_c: zero the weight-side values whose
             // k lies at or beyond the end of the tile's window (XTR, the tile's last slices)
-            auto load_block = [&](bf16x8 (&wf)[FN], bf16x8 (&xf)[FM], int slot_i, int sub, int item, auto mask_c) {
+            auto load_block = [&](bf16x8 (&wf)[FN], bf16x8 (&xf)[FM], int slot_i, int sub, int item, auto mask_c, auto act_c) {
                 constexpr bool MASK = XTR && decltype(mask_c)::value;
+                constexpr int ACT = decltype(act_c)::value;     // row blocks that are multiplied
                 const uint8_t* sx = smem + slot_i * TL::STAGE_BYTES;
                 const uint8_t* sw = sx + BM * 64;
                 const int chunk = 2 * sub + khalf;
@@ -1683,7 +1704,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                     else wf[fn] = *reinterpret_cast<const bf16x8*>(sw + lds_off64(wfrag_row[fn], chunk));
                 }
 #pragma unroll
-                for (int fm = 0; fm < FM; ++fm) {
+                for (int fm = 0; fm < ACT; ++fm) {
                     if constexpr (XTR) xf[fm] = read_tr(sx + xtr_off[fm] + sub * 4096);
                     else xf[fm] = *reinterpret_cast<const bf16x8*>(sx + lds_off64(xfrag_row[fm], chunk));
                 }
@@ -1706,16 +1727,20 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             // the 8 MFMAs of a block, with the L parts of the pair being issued between them
             // when DMA is set.  The two waves of a SIMD (w and w + NW/2) issue in different
             // blocks, so that while one sits in its VMEM issue the other feeds the MFMA pipe.
-            auto mma_block = [&](const bf16x8 (&wf)[FN], const bf16x8 (&xf)[FM], auto dma_c) {
+            auto mma_block = [&](const bf16x8 (&wf)[FN], const bf16x8 (&xf)[FM], auto dma_c, auto act_c) {
                 constexpr bool DMA = decltype(dma_c)::value;
-                constexpr int NM = FN * FM, EVERY = NM / L;
+                constexpr int ACT = decltype(act_c)::value;
+                constexpr int NM = FN * ACT;
+                static_assert(NM % L == 0 || L % NM == 0, "DMA parts must spread evenly over the MFMAs");
+                constexpr int PER = L >= NM ? L / NM : 1, EVERY = L >= NM ? 1 : NM / L;
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
-                    const int fn = m / FM, fm = m % FM;
+                    const int fn = m / ACT, fm = m % ACT;
                     acc[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0);
                     if (DMA && (m + 1) % EVERY == 0) {
                         __builtin_amdgcn_sched_barrier(0);
-                        issue_part((m + 1) / EVERY - 1);
+#pragma unroll
+                        for (int q = 0; q < PER; ++q) issue_part(((m + 1) / EVERY - 1) * PER + q);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -1734,25 +1759,27 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             // (store16_uniform_base) and followed by a wait that leaves at most that many operations
             // in flight, i.e. nothing older than the stores.  The counted wait here would sit out the
             // stores' own round trip instead (one counter serves loads and stores, in order).
-            auto double_step = [&](auto half_c, auto last_c, auto mask_c, bool skip_wait) __attribute__((always_inline)) {
+            auto double_step = [&](auto half_c, auto last_c, auto mask_c, auto act_c, bool skip_wait) __attribute__((always_inline)) {
                 constexpr int HALF = decltype(half_c)::value;
+                constexpr int ACT = decltype(act_c)::value;
                 constexpr bool LAST = decltype(last_c)::value;   // last of the tile: no fragments kept over the epilogue
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
                 const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
                 auto interleave = [&]() {   // one fragment read in the shadow of every MFMA
+                    static_assert(ACT * FN >= ACT + FN, "more fragment reads than MFMAs to hide them under");
 #pragma unroll
-                    for (int i = 0; i < FM + FN; ++i) {
+                    for (int i = 0; i < ACT + FN; ++i) {
                         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                         __builtin_amdgcn_sched_group_barrier(0x100, (WTR || XTR) ? 2 : 1, 0);
                     }
-                    __builtin_amdgcn_sched_group_barrier(0x008, FM * FN - (FM + FN), 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, ACT * FN - (ACT + FN), 0);
                 };
-                load_block(wfb, xfb, cslot, 1, kitem, mask_c);
-                mma_block(wfa, xfa, std::false_type{});
+                load_block(wfb, xfb, cslot, 1, kitem, mask_c, act_c);
+                mma_block(wfa, xfa, std::false_type{}, act_c);
                 interleave();
                 __builtin_amdgcn_sched_barrier(0);
-                load_block(wfa, xfa, s1, 0, kitem + 1, mask_c);
-                mma_block(wfb, xfb, std::false_type{});
+                load_block(wfa, xfa, s1, 0, kitem + 1, mask_c, act_c);
+                mma_block(wfb, xfb, std::false_type{}, act_c);
                 interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 barrier();                  // B
@@ -1767,9 +1794,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                     part_wkoff += ikt >= split_kt ? split_w : 0;
                 }
                 ikt += 2;
-                load_block(wfb, xfb, s1, 1, kitem + 1, mask_c);
+                load_block(wfb, xfb, s1, 1, kitem + 1, mask_c, act_c);
                 if constexpr (HALF == 0) __builtin_amdgcn_sched_barrier(0);
-                mma_block(wfa, xfa, std::integral_constant<bool, HALF == 0>{});
+                mma_block(wfa, xfa, std::integral_constant<bool, HALF == 0>{}, act_c);
                 if constexpr (HALF != 0) interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 // pair (c+2, c+3) is older than the 2L instructions the first half just issued
@@ -1778,9 +1805,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                     else wait_vmcnt<0>();
                 }
                 barrier();                  // A'
-                if (!LAST) load_block(wfa, xfa, s2, 0, kitem + 2, mask_c);
+                if (!LAST) load_block(wfa, xfa, s2, 0, kitem + 2, mask_c, act_c);
                 if constexpr (HALF == 1 || LAST) __builtin_amdgcn_sched_barrier(0);
-                mma_block(wfb, xfb, std::integral_constant<bool, HALF == 1>{});
+                mma_block(wfb, xfb, std::integral_constant<bool, HALF == 1>{}, act_c);
                 if constexpr (HALF != 1 && !LAST) interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 cslot = s2;
@@ -1788,11 +1815,11 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             // the issue side runs 4 items ahead: it enters the next tile 4 items before the end;
             // the last two double steps hold the end of an XTR tile's window and mask it
-            auto tile_steps = [&](auto half_c) __attribute__((always_inline)) {
+            auto tile_steps = [&](auto half_c, auto act_c) __attribute__((always_inline)) {
                 const int tile_kt = KWIN ? cur.kt : KT;
                 bool landed = tile_i > 0;       // the first step's pair landed before the previous epilogue's stores
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) {
-                    double_step(half_c, std::false_type{}, std::false_type{}, landed);
+                    double_step(half_c, std::false_type{}, std::false_type{}, act_c, landed);
                     landed = false;
 #ifdef FMOE_TRACE
                     if (kt < 8) FMOE_TRACE_STAMP(6 + kt / 2);
@@ -1801,17 +1828,23 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 FMOE_TRACE_STAMP(10);
                 enter_next();
                 ikt = 0;
-                double_step(half_c, std::false_type{}, std::true_type{}, landed);
+                double_step(half_c, std::false_type{}, std::true_type{}, act_c, landed);
                 FMOE_TRACE_STAMP(11);
-                double_step(half_c, std::true_type{}, std::true_type{}, false);
+                double_step(half_c, std::true_type{}, std::true_type{}, act_c, false);
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
                 wait_vmcnt<2 * L>();
                 barrier();
             }
-            load_block(wfa, xfa, cslot, 0, 0, std::true_type{});
-            if (wave < NW / 2) tile_steps(std::integral_constant<int, 0>{});
-            else tile_steps(std::integral_constant<int, 1>{});
+            load_block(wfa, xfa, cslot, 0, 0, std::true_type{}, std::integral_constant<int, FM>{});
+            const bool sparse = SPARSE && cur.rows_valid <= BM / 2;
+            if (wave < NW / 2) {
+                if (sparse) tile_steps(std::integral_constant<int, 0>{}, std::integral_constant<int, SPARSE ? ACT_SPARSE : FM>{});
+                else tile_steps(std::integral_constant<int, 0>{}, std::integral_constant<int, FM>{});
+            } else {
+                if (sparse) tile_steps(std::integral_constant<int, 1>{}, std::integral_constant<int, SPARSE ? ACT_SPARSE : FM>{});
+                else tile_steps(std::integral_constant<int, 1>{}, std::integral_constant<int, FM>{});
+            }
         } else if constexpr (PAIR) {
             // e4m3: the same double step; an item is one 32x32x64 MFMA deep, so its two blocks
             // split the activation fragments instead of K: block 0 reads both weight
@@ -1836,9 +1869,18 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 #pragma unroll
                 for (int fm = 0; fm < HM; ++fm) xh[fm] = load_frag(sx, xfrag_row[HM + fm]);
             };
-            auto mma_block = [&](const i32x8 (&wf)[FN], const i32x8 (&xh)[HM], int fm0, auto dma_c) {
+            // skip_c: the block's row blocks hold no valid row (sparse tile); only its share of the
+            // DMA issue is left
+            auto mma_block = [&](const i32x8 (&wf)[FN], const i32x8 (&xh)[HM], int fm0, auto dma_c, auto skip_c) {
                 constexpr bool DMA = decltype(dma_c)::value;
                 constexpr int NM = FN * HM;
+                if constexpr (decltype(skip_c)::value) {
+                    if constexpr (DMA) {
+#pragma unroll
+                        for (int q = 0; q < L; ++q) issue_part(q);
+                    }
+                    return;
+                }
                 static_assert(NM % L == 0 || L % NM == 0, "DMA parts must spread evenly over the MFMAs");
                 constexpr int PER = L >= NM ? L / NM : 1, EVERY = L >= NM ? 1 : NM / L;
 #pragma unroll
@@ -1859,18 +1901,20 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 __builtin_amdgcn_s_barrier();
                 asm volatile("" ::: "memory");
             };
-            auto double_step = [&](auto half_c, auto last_c, bool skip_wait) __attribute__((always_inline)) {   // skip_wait: as in the bf16 loop
+            auto double_step = [&](auto half_c, auto last_c, auto sparse_c, bool skip_wait) __attribute__((always_inline)) {   // skip_wait: as in the bf16 loop
                 constexpr int HALF = decltype(half_c)::value;
                 constexpr bool LAST = decltype(last_c)::value;
+                constexpr bool SP = decltype(sparse_c)::value;  // row blocks HM.. are not multiplied
+                constexpr std::false_type full{};
                 const int s1 = cslot + 1 == STAGES ? 0 : cslot + 1;
                 const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
-                load_x1(qx1, cslot);
+                if (!SP) load_x1(qx1, cslot);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwa, qx0, 0, std::false_type{});
+                mma_block(qwa, qx0, 0, std::false_type{}, full);
                 __builtin_amdgcn_sched_barrier(0);
                 load_w_x0(qwb, qx0, s1);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwa, qx1, HM, std::false_type{});
+                mma_block(qwa, qx1, HM, std::false_type{}, sparse_c);
                 __builtin_amdgcn_sched_barrier(0);
                 barrier();                  // B
                 part_a = lds_base + islot * TL::STAGE_BYTES;    // pair (c+4, c+5)
@@ -1880,9 +1924,9 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 part_koff = (int64_t)ikt * xstep;
                 part_wkoff = WTR ? (int64_t)ikt * wstep : part_koff;
                 ikt += 2;
-                load_x1(qx1, s1);
+                if (!SP) load_x1(qx1, s1);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwb, qx0, 0, std::integral_constant<bool, HALF == 0>{});
+                mma_block(qwb, qx0, 0, std::integral_constant<bool, HALF == 0>{}, full);
                 __builtin_amdgcn_sched_barrier(0);
                 if (!skip_wait) {
                     if (HALF == 0) wait_vmcnt<2 * L>();
@@ -1891,11 +1935,11 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 barrier();                  // A'
                 if (!LAST) load_w_x0(qwa, qx0, s2);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwb, qx1, HM, std::integral_constant<bool, HALF == 1>{});
+                mma_block(qwb, qx1, HM, std::integral_constant<bool, HALF == 1>{}, sparse_c);
                 __builtin_amdgcn_sched_barrier(0);
                 cslot = s2;
             };
-            auto tile_steps = [&](auto half_c) __attribute__((always_inline)) {
+            auto tile_steps = [&](auto half_c, auto sparse_c) __attribute__((always_inline)) {
                 const int tile_kt = KWIN ? cur.kt : KT;
                 // (whatever the compiler still counts as pending from the tile's set-up or the last
                 // epilogue, spill reloads and the row-index loads, is settled by the counted wait at
@@ -1903,7 +1947,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 // drains the LDS-DMA stream, which the compiler cannot see, on every iteration)
                 bool landed = tile_i > 0;
                 for (int kt = 0; kt < tile_kt - 4; kt += 2) {
-                    double_step(half_c, std::false_type{}, landed);
+                    double_step(half_c, std::false_type{}, sparse_c, landed);
                     landed = false;
 #ifdef FMOE_TRACE
                     if (kt < 8) FMOE_TRACE_STAMP(6 + kt / 2);
@@ -1912,17 +1956,23 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 FMOE_TRACE_STAMP(10);
                 enter_next();
                 ikt = 0;
-                double_step(half_c, std::false_type{}, landed);
+                double_step(half_c, std::false_type{}, sparse_c, landed);
                 FMOE_TRACE_STAMP(11);
-                double_step(half_c, std::true_type{}, false);
+                double_step(half_c, std::true_type{}, sparse_c, false);
             };
             if (tile_i == 0) {              // pair 0 has landed everywhere
                 wait_vmcnt<2 * L>();
                 barrier();
             }
             load_w_x0(qwa, qx0, cslot);
-            if (wave < NW / 2) tile_steps(std::integral_constant<int, 0>{});
-            else tile_steps(std::integral_constant<int, 1>{});
+            const bool sparse = SPARSE && cur.rows_valid <= BM / 2;
+            if (wave < NW / 2) {
+                if (sparse) tile_steps(std::integral_constant<int, 0>{}, std::integral_constant<bool, SPARSE>{});
+                else tile_steps(std::integral_constant<int, 0>{}, std::false_type{});
+            } else {
+                if (sparse) tile_steps(std::integral_constant<int, 1>{}, std::integral_constant<bool, SPARSE>{});
+                else tile_steps(std::integral_constant<int, 1>{}, std::false_type{});
+            }
         } else {
             for (int kt = 0; kt < KT; ++kt) {
                 if (c > landed) {
@@ -1953,11 +2003,11 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             rows_to_offsets(ridx_next, xoff_next);  // of the tile after the next one
         };
 #ifdef FMOE_TRACE
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR, ROW_IL>(
             p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane, convert_rows,
             (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2)) ? tstamp + 12 : nullptr);
 #else
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR, ROW_IL>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                                 done.rows_valid, wm, wn, lane, convert_rows);
 #endif
 #ifdef FMOE_TRACE

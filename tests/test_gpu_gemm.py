@@ -302,6 +302,52 @@ def test_ring_kernel_shapes(L, E, K, Din, Dout, epi):
         assert_bf16_close(out, ref, rtol=1.6e-2, atol=1e-2, what=f"ring swiglu {L},{E},{K},{Din},{Dout}")
 
 
+@pytest.mark.parametrize("epi,fp8", [("plain", False), ("swiglu", False), ("plain", True)])
+def test_ring_kernel_tiles_with_few_valid_rows(epi, fp8):
+    """Experts whose last (or only) 256-row tile ends at, just before and just after every 32-row
+    block boundary: tiles that end in their first half run the ring kernel's shortened main loop,
+    and the two wave rows share a tile's row blocks alternately.  Against the oracle, and the plan
+    must say RING."""
+    from fast_moe_amd.kernels import moe, moe_fp8
+    from fast_moe_amd.kernels.hip import _lib, ops
+    lens = [1, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 160, 191, 193, 255, 256, 257, 288, 320, 383, 384, 385,
+            511, 513, 640, 0, 769, 2048 + 17, 3000]
+    E, Din, Dout = len(lens), 192, 320
+    g = torch.Generator().manual_seed(7)
+    experts = torch.repeat_interleave(torch.arange(E), torch.tensor(lens))
+    topk = experts[torch.randperm(experts.numel(), generator=g)].view(-1, 1)
+    L = topk.shape[0]
+    meta = o_routing.routing_metadata(topk.numpy(), E)
+    offsets = torch.from_numpy(meta["offsets"])
+    index = torch.from_numpy(meta["gate_index"]).view(-1, 1)
+    assert (offsets[1:] - offsets[:-1]).tolist() == lens
+    x = randn((L, Din), 1)
+    w = weights(E, Din, Dout, 2, False, scale=Din ** -0.5)
+    b = randn((E, Dout), 3)
+    # (the plan of the bf16 descriptor of this shape; the e4m3 one differs in the operand type only)
+    assert ops.grouped_gemm(dev(offsets), dev(x), dev(w), total_rows=L, row_index=dev(index).view(-1), index_div=1,
+                            plan_only=True) == _lib.PLAN_RING
+    with torch.no_grad():
+        if fp8:
+            ref = o_fp8.index_select_jagged_bmm_fp8(offsets, index, x, w, b)
+            out = moe_fp8.index_select_jagged_bmm(0, dev(offsets), dev(index), dev(x), dev(w), dev(b), fp8=True)
+        elif epi == "plain":
+            ref = o_moe.index_select_jagged_bmm(offsets, index, x.float(), w.float(), b.float())
+            out = moe.index_select_jagged_bmm(0, dev(offsets), dev(index), dev(x), dev(w), dev(b))
+        else:
+            wp = weights(E, Din, Dout, 5, False, scale=Din ** -0.5)
+            ref = o_moe.index_select_jagged_bmm_swiglu(offsets, index, x.float(), w.float(), b.float(),
+                                                       wp.float(), None)
+            out = moe.index_select_jagged_bmm_swiglu(0, dev(offsets), dev(index), dev(x), dev(w), dev(b),
+                                                     dev(wp), None)
+    # every expert on its own, so that a failure names the row count it happens at
+    for e, n in enumerate(lens):
+        lo = int(offsets[e])
+        if n:
+            assert_bf16_close(out[lo:lo + n], ref[lo:lo + n], rtol=3e-2 if fp8 else 1.6e-2, atol=3e-2 if fp8 else 1e-2,
+                              what=f"expert {e} with {n} rows ({epi}, fp8={fp8})")
+
+
 def test_ring_kernel_is_deterministic_and_ignores_garbage_offsets():
     """Two launches give identical bits; offsets outside [0, R] are clamped instead of followed."""
     from fast_moe_amd.kernels.hip import ops
