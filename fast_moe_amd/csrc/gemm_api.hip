@@ -42,7 +42,7 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
                  "fmoe_grouped_gemm: operands must be bf16, e4m3 or fp32 (got dtype %d)", d->a_dtype);
     FMOE_REQUIRE(d->out_dtype == (d->a_dtype == FMOE_F32 ? FMOE_F32 : FMOE_BF16),
                  "fmoe_grouped_gemm: output must be bf16 (fp32 for fp32 operands)");
-    FMOE_REQUIRE(d->epilogue >= FMOE_EPI_NONE && d->epilogue <= FMOE_EPI_SWIGLU,
+    FMOE_REQUIRE(d->epilogue >= FMOE_EPI_NONE && d->epilogue <= FMOE_EPI_GATED,
                  "fmoe_grouped_gemm: unknown epilogue %d", d->epilogue);
     if (d->total_rows == 0) return FMOE_OK;     // sel stays -1
     FMOE_REQUIRE(d->offsets && d->a && d->b && d->out, "fmoe_grouped_gemm: NULL tensor pointer");
@@ -58,9 +58,17 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     const bool f32 = d->a_dtype == FMOE_F32;
     const bool swiglu = d->epilogue == FMOE_EPI_SWIGLU;
     if (swiglu) FMOE_REQUIRE(d->b2 != nullptr, "fmoe_grouped_gemm: SWIGLU needs b2");
-    FMOE_REQUIRE((d->aux == nullptr) == (d->aux2 == nullptr), "fmoe_grouped_gemm: aux and aux2 come together");
+    const bool gated = d->epilogue == FMOE_EPI_GATED;
+    if (gated) {
+        FMOE_REQUIRE(d->aux && !d->aux2, "fmoe_grouped_gemm: GATED reads its gate from aux (aux2 stays NULL)");
+        if (d->a_dtype != FMOE_BF16)
+            return fmoe::fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: the GATED epilogue is built for bf16 operands");
+        FMOE_REQUIRE(!d->a_silu && !d->out2 && !d->a2, "fmoe_grouped_gemm: GATED goes without a_silu, out2 and a2");
+    } else {
+        FMOE_REQUIRE((d->aux == nullptr) == (d->aux2 == nullptr), "fmoe_grouped_gemm: aux and aux2 come together");
+    }
     if (d->aux) {
-        FMOE_REQUIRE(swiglu, "fmoe_grouped_gemm: aux outputs are the SWIGLU pre-activations");
+        FMOE_REQUIRE(swiglu || gated, "fmoe_grouped_gemm: aux outputs are the SWIGLU pre-activations");
         FMOE_REQUIRE(d->aux_stride_row >= d->n, "fmoe_grouped_gemm: aux row stride %lld < n %d",
                      (long long)d->aux_stride_row, d->n);
     }
@@ -134,9 +142,10 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     const int64_t stride_cap = (int64_t)1 << 25;
     p.vec_store = (d->n % vec_cols == 0) && (d->out_stride_row % vec_cols == 0) && aligned16(d->out) &&
                   d->out_stride_row < stride_cap &&
-                  (!d->aux || ((d->aux_stride_row % vec_cols == 0) && aligned16(d->aux) && aligned16(d->aux2) &&
-                               d->aux_stride_row < stride_cap));
+                  (!d->aux || gated || ((d->aux_stride_row % vec_cols == 0) && aligned16(d->aux) && aligned16(d->aux2) &&
+                                        d->aux_stride_row < stride_cap));
 
+    p.gate_vec = gated && (reinterpret_cast<uintptr_t>(d->aux) % 8 == 0) && d->aux_stride_row % 4 == 0;
     p.scale_vec = fp8 && d->n >= 4 && d->n % 4 == 0 && aligned16(d->b_scale) && (!d->b2_scale || aligned16(d->b2_scale));
     const int esize = fp8 ? 1 : (f32 ? 4 : 2);
     const int chunk = 16 / esize;

@@ -13,6 +13,7 @@ int run_gemm_bf16(GemmParams& p, int epilogue, bool a_silu, int sel, hipStream_t
         case FMOE_EPI_NONE: return dispatch_tile<kDtBf16, FMOE_EPI_NONE, false>(p, sel, stream);
         case FMOE_EPI_SILU: return dispatch_tile<kDtBf16, FMOE_EPI_SILU, false>(p, sel, stream);
         case FMOE_EPI_SWIGLU: return dispatch_tile<kDtBf16, FMOE_EPI_SWIGLU, false>(p, sel, stream);
+        case FMOE_EPI_GATED: return dispatch_tile<kDtBf16, FMOE_EPI_GATED, false>(p, sel, stream);
     }
     return fail(FMOE_ERR_ARGUMENT, "fmoe_grouped_gemm: unknown epilogue %d", epilogue);
 }

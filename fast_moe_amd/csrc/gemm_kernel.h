@@ -73,6 +73,7 @@ struct GemmParams {
     int n_tiles;
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
     int scale_vec;                      // e4m3: 16-byte loads of 4 weight scales are legal
+    int gate_vec;                       // GATED: 8-byte loads of 4 gate values are legal
     const int64_t* k_window;            // [E+1] per-expert contraction range, or null
     int k_window_multiple;              // every window is a multiple of this and at least twice it (0: unknown)
     uint16_t* aux;                      // SWIGLU: the two pre-activations, or null
@@ -226,6 +227,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                               int lane, AfterStores after_stores = AfterStores(),
                                               uint64_t* ets = nullptr) {
     constexpr bool SWIGLU = EPI == FMOE_EPI_SWIGLU;
+    constexpr bool GATED = EPI == FMOE_EPI_GATED;   // out = silu(gate from p.aux) * (acc + bias); bf16 operands
+    static_assert(!(GATED && FP8), "the gated epilogue is built for bf16 operands");
     constexpr int FN_OUT = SWIGLU ? FN / 2 : FN;
     // (ring kernel: everything derived from the lane number below is recomputed per tile; as
     // tile-loop invariants the compiler keeps such values in registers across the main loop, or
@@ -356,7 +359,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     auto run = [&](auto has_bias_c, auto has_aux_c) {
         constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
         constexpr bool HAS_AUX = SWIGLU && decltype(has_aux_c)::value;   // keep the pre-activations (training)
-        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && FN_OUT == 2;   // plain and SiLU epilogues of the ring kernel, bf16 and e4m3
+        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && !GATED && FN_OUT == 2;   // plain and SiLU epilogues of the ring kernel, bf16 and e4m3
         // per-column biases of this lane, indexed like rsw
         float bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
         // with a bias, at least one of the two pointers is set: both loads go through a valid
@@ -481,12 +484,47 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                 __builtin_amdgcn_sched_barrier(0);
                 continue;
             }
+            // GATED: the row block's gate values, all loads of the block issued together (one memory
+            // latency per 32-row block; loaded where they are used, every group of 8 waits out its own)
+            u32x2 graw[FN_OUT][2][2];
+            if constexpr (GATED) {
+                const int64_t grow = row0 + (row_ok[fm] ? frag_row(fm) + (lane & 31) : 0);
+                const uint16_t* gp_row = p.aux + grow * p.aux_stride;
+#pragma unroll
+                for (int fn = 0; fn < FN_OUT; ++fn)
+#pragma unroll
+                    for (int gp = 0; gp < 2; ++gp)
+#pragma unroll
+                        for (int q = 0; q < 2; ++q) {
+                            const int n = col0 + fn * 32 + 16 * gp + 8 * q + 4 * khalf;
+                            if (p.gate_vec && n + 3 < p.N) {
+                                graw[fn][gp][q] = *reinterpret_cast<const u32x2*>(gp_row + n);
+                            } else {
+                                uint32_t e[4];
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) e[j] = n + j < p.N ? (uint32_t)gp_row[n + j] : 0u;
+                                graw[fn][gp][q] = u32x2{e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
+                            }
+                        }
+            }
 #pragma unroll
             for (int fn = 0; fn < FN_OUT; ++fn) {
 #pragma unroll
                 for (int gp = 0; gp < 2; ++gp) {
                     const int nq = col0 + fn * 32 + 16 * gp;
                     float o[2][4], pg[2][4], pu[2][4];
+                    // GATED: this lane's 2 x 4 gate values (its row, columns nq + 8q + 4*khalf + 0..3)
+                    float gate[2][4];
+                    if constexpr (GATED) {
+#pragma unroll
+                        for (int q = 0; q < 2; ++q) {
+                            const u32x2 g2 = graw[fn][gp][q];
+                            gate[q][0] = __uint_as_float(g2[0] << 16);
+                            gate[q][1] = __uint_as_float(g2[0] & 0xffff0000u);
+                            gate[q][2] = __uint_as_float(g2[1] << 16);
+                            gate[q][3] = __uint_as_float(g2[1] & 0xffff0000u);
+                        }
+                    }
                     // two columns at a time: one conversion instruction rounds a pair
 #pragma unroll
                     for (int q = 0; q < 2; ++q)
@@ -528,6 +566,12 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                     }
                                     rbf2(ua, ub);
                                 }
+                                if constexpr (GATED) {      // the product so far is the factor, the gate the argument
+                                    ua = ya;
+                                    ub = yb;
+                                    ya = gate[q][j];
+                                    yb = gate[q][j + 1];
+                                }
                             }
                             pg[q][j] = ya;
                             pg[q][j + 1] = yb;
@@ -537,7 +581,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                 ya = fast_silu_f32(ya);
                                 yb = fast_silu_f32(yb);
                             }
-                            if (SWIGLU) {
+                            if (SWIGLU || GATED) {
                                 ya = fast_silu_f32(ya);
                                 yb = fast_silu_f32(yb);
                                 rbf2(ya, yb);

@@ -13,7 +13,7 @@ _PKG_DIR = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__fil
 LIB_PATH = os.path.join(_PKG_DIR, "libfastmoe_hip.so")
 
 FMOE_F32, FMOE_BF16, FMOE_E4M3 = 0, 1, 2
-EPI_NONE, EPI_SILU, EPI_SWIGLU = 0, 1, 2
+EPI_NONE, EPI_SILU, EPI_SWIGLU, EPI_GATED = 0, 1, 2, 3
 PLAN_NONE, PLAN_RING, PLAN_STAGED, PLAN_STAGED_SHORT, PLAN_ELEMENT = -1, 0, 1, 2, 3
 
 # every symbol include/fast_moe_amd.h declares

@@ -11,7 +11,7 @@ from typing import Dict, Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import EPI_NONE, EPI_SILU, EPI_SWIGLU, FMOE_BF16, FMOE_E4M3, FMOE_F32, GemmDesc
+from ._lib import EPI_GATED, EPI_NONE, EPI_SILU, EPI_SWIGLU, FMOE_BF16, FMOE_E4M3, FMOE_F32, GemmDesc
 
 _DTYPE_CODE = {torch.float32: FMOE_F32, torch.bfloat16: FMOE_BF16}
 FP8_DTYPE = torch.float8_e4m3fn
@@ -273,11 +273,13 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  k_window: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                  k_window_multiple: int = 0,
                  aux: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                 gate: Optional[torch.Tensor] = None,
                  plan_only: bool = False) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
     strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
     [total_rows, N] in bf16 (fp32 for fp32 operands).  ``aux`` = two tensors like the output
-    that receive the SWIGLU pre-activations.  ``plan_only``: launch nothing and return the
+    that receive the SWIGLU pre-activations.  ``gate`` (bf16 [total_rows, N], with
+    ``epilogue=EPI_GATED``): the result is ``silu(gate) * (A B + bias)``.  ``plan_only``: launch nothing and return the
     _lib.PLAN_* code of the kernel this call would run (fmoe_grouped_gemm_plan)."""
     dev = _need_cuda("grouped_gemm", offsets, a, b, row_index, bias, b2, bias2, a_scale, b_scale, b2_scale)
     fp8 = a.dtype == FP8_DTYPE
@@ -321,6 +323,15 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                     or t.stride(0) != aux[0].stride(0)):
                 raise ValueError(f"grouped_gemm: aux tensors must be {out_dtype} [{total_rows}, {N}] with "
                                  "contiguous rows and one row stride")
+    if (gate is not None) != (epilogue == EPI_GATED):
+        raise ValueError("grouped_gemm: gate and EPI_GATED come together")
+    if gate is not None:
+        if a.dtype != torch.bfloat16:
+            raise NotImplementedError("grouped_gemm: the gated epilogue is built for bf16 operands")
+        if (tuple(gate.shape) != (total_rows, N) or gate.dtype != out_dtype or gate.device != dev
+                or gate.stride(1) != 1 or aux is not None):
+            raise ValueError(f"grouped_gemm: gate must be {out_dtype} [{total_rows}, {N}] with contiguous rows "
+                             "(and no aux outputs)")
     if total_rows == 0:
         return _lib.PLAN_NONE if plan_only else out
 
@@ -373,6 +384,8 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.k_window_multiple = k_window_multiple if k_window is not None else 0
     if aux is not None:
         d.aux, d.aux2, d.aux_stride_row = aux[0].data_ptr(), aux[1].data_ptr(), aux[0].stride(0)
+    if gate is not None:
+        d.aux, d.aux_stride_row = gate.data_ptr(), gate.stride(0)
     lib = _lib.load()
     # N-contiguous weights of a useful size that only the element-load kernel would read in
     # place (correct, but an order of magnitude slower): one transposing copy buys a streaming kernel

@@ -23,7 +23,7 @@ import torch
 
 from .hip import autograd as _ag
 from .hip import ops
-from .hip._lib import EPI_NONE, EPI_SWIGLU
+from .hip._lib import EPI_GATED, EPI_NONE, EPI_SWIGLU
 from .utils import KernelType, require_hip_kernel
 
 
@@ -157,7 +157,8 @@ def index_select_jagged_gating_bmm(
     kernel: KernelType = KernelType.HIP,
 ) -> torch.Tensor:
     """kernels/moe.py:192-233.  ``silu(A Wa + ba) * (B Wb + bb)``; one fused kernel when A is B,
-    otherwise two GEMMs and an element-wise kernel."""
+    otherwise two GEMMs, the second of which multiplies by the SiLU of the first one's result in
+    its epilogue (bf16; fp32: two GEMMs and an element-wise kernel)."""
     require_hip_kernel(kernel, "index_select_jagged_gating_bmm")
     assert (index.ndim == 2 and index.shape[0] == jagged_a.shape[0] == jagged_b.shape[0]
             and jagged_a.shape == jagged_b.shape and weight_a.shape == weight_b.shape)
@@ -169,6 +170,9 @@ def index_select_jagged_gating_bmm(
                                                     bias_a, bias_b)
     alpha = ops.grouped_gemm(offsets, jagged_a, weight_a, total_rows=index.numel(), row_index=index,
                              index_div=index.shape[-1], bias=bias_a)
+    if jagged_a.dtype == torch.bfloat16 and index.numel() > 0:
+        return ops.grouped_gemm(offsets, jagged_b, weight_b, total_rows=index.numel(), row_index=index,
+                                index_div=index.shape[-1], bias=bias_b, epilogue=EPI_GATED, gate=alpha)
     beta = ops.grouped_gemm(offsets, jagged_b, weight_b, total_rows=index.numel(), row_index=index,
                             index_div=index.shape[-1], bias=bias_b)
     return ops.silu_mul(alpha, beta)

@@ -36,7 +36,13 @@ enum fmoe_dtype {
 enum fmoe_epilogue {
     FMOE_EPI_NONE = 0,  /* out = acc + bias                                  */
     FMOE_EPI_SILU = 1,  /* out = silu(round(acc + bias))                     */
-    FMOE_EPI_SWIGLU = 2 /* out = silu(round(acc + bias)) * round(acc2 + bias2) */
+    FMOE_EPI_SWIGLU = 2, /* out = silu(round(acc + bias)) * round(acc2 + bias2) */
+    FMOE_EPI_GATED = 3   /* out = round(silu(gate)) * round(acc + bias), gate = the [total_rows, n]
+                            bf16 tensor in desc.aux (an input here): the second GEMM of the gating
+                            operator whose two GEMMs read different inputs, multiplied into the
+                            first one's result where it is produced (the one kernel with two input
+                            pointers of kernels/triton/triton_moe.py:2993-3159 as two launches
+                            without the product's round trip); bf16 operands only              */
 };
 
 enum fmoe_status {
@@ -227,7 +233,8 @@ typedef struct fmoe_gemm_desc {
                                 the k columns of A and B)                              */
     int32_t k_slack_rows;   /* with a_stride_k: rows readable behind the last k row of A and of
                                 B (128 or more; what they hold does not matter)      */
-    void* aux;              /* NULL, or with FMOE_EPI_SWIGLU [total_rows, n] in out_dtype:  */
+    void* aux;              /* with FMOE_EPI_GATED: the gate, read (aux2 NULL).  Otherwise
+                                NULL, or with FMOE_EPI_SWIGLU [total_rows, n] in out_dtype:  */
     void* aux2;             /* receive A x B + bias (aux) and A x B2 + bias2 (aux2), the
                                 two pre-activations the backward pass needs (the ALPHA and
                                 BETA outputs of kernels/triton/triton_moe.py:2316-2345) */

@@ -111,6 +111,55 @@ def test_swiglu_and_gating(L, E, K, Din, Dout, bias, contiguous):
     assert_bf16_close(out_two, ref2, rtol=1.6e-2, atol=2e-2, what="gating")
 
 
+@pytest.mark.parametrize("L,E,K,Din,Dout,bias,contiguous", [
+    (8192, 8, 2, 512, 384, True, False),       # LDS-ring kernel
+    (8192, 8, 2, 512, 384, False, True),       # the same with [E, K, N]-contiguous weights read in place
+    (4096, 16, 4, 256, 200, True, False),      # ring, N tail: 200 columns of a 256-column tile
+    (600, 4, 2, 128, 136, True, False),        # register-staged kernel, tall tile
+    (64, 16, 2, 128, 64, False, False),        # register-staged kernel, 64-row tile
+    (100, 8, 2, 24, 40, True, True),           # element loads and element stores
+    (300, 4, 2, 64, 36, True, False),          # gate rows that start off 8-byte boundaries (N = 36)
+])
+def test_two_input_gating_multiplies_in_the_second_gemm(L, E, K, Din, Dout, bias, contiguous):
+    """index_select_jagged_gating_bmm with two different inputs: the second GEMM's epilogue multiplies
+    by the SiLU of the first one's result (no element-wise pass, no second [rows, N] round trip).
+    Against the oracle, and against the three-launch composition (which differs by the SiLU's last
+    fp32 bits before its bf16 rounding: the element-wise kernel divides, the epilogue uses the
+    hardware reciprocal)."""
+    from fast_moe_amd.kernels import moe
+    from fast_moe_amd.kernels.hip import ops
+    r = make_routing(L, E, K, seed=L + 3)
+    x, x2 = randn((L, Din), 1), randn((L, Din), 4)
+    w, wp = (weights(E, Din, Dout, s, contiguous, scale=Din ** -0.5) for s in (2, 5))
+    b = randn((E, Dout), 3) if bias else None
+    bp = randn((E, Dout), 6) if bias else None
+    f = lambda t: None if t is None else t.float()
+    ref = o_moe.index_select_jagged_gating_bmm(r["offsets"], r["index"], f(x), f(x2), f(w), f(wp), f(b), f(bp))
+    off, idx = dev(r["offsets"]), dev(r["index"])
+    calls = []
+    real = ops.silu_mul
+    ops.silu_mul = lambda *a, **k: calls.append(1) or real(*a, **k)
+    try:
+        with torch.no_grad():
+            out = moe.index_select_jagged_gating_bmm(0, off, idx, dev(x), dev(x2), dev(w), dev(b), dev(wp), dev(bp))
+    finally:
+        ops.silu_mul = real
+    assert not calls, "the element-wise pass ran"
+    assert_bf16_close(out, ref, rtol=1.6e-2, atol=2e-2, what="gating, two inputs")
+    kw = dict(total_rows=L * K, row_index=idx, index_div=K)
+    alpha = ops.grouped_gemm(off, dev(x), dev(w), bias=dev(b), **kw)
+    beta = ops.grouped_gemm(off, dev(x2), dev(wp), bias=dev(bp), **kw)
+    three = ops.silu_mul(alpha, beta)
+    diff = (out.view(torch.int16).int() - three.view(torch.int16).int()).abs()
+    # (one bf16 step of the rounded SiLU is up to two steps of the rounded product)
+    assert int(diff.max()) <= 2 and float((diff != 0).float().mean()) < 2e-3, (int(diff.max()), float((diff != 0).float().mean()))
+    # a gate tensor that is a column slice of a wider one (row stride > N)
+    wide = torch.zeros((L * K, Dout + 12), dtype=BF16, device="cuda")
+    wide[:, 4:4 + Dout] = alpha
+    sliced = ops.grouped_gemm(off, dev(x2), dev(wp), bias=dev(bp), epilogue=3, gate=wide[:, 4:4 + Dout], **kw)
+    assert torch.equal(sliced, out)
+
+
 def test_3d_variant():
     from fast_moe_amd.kernels import moe
     L, E, K, Din, Dout = 200, 4, 2, 8, 4
