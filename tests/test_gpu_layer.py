@@ -209,3 +209,51 @@ def test_layer_forward_replays_from_a_captured_graph():
                 torch.cuda.synchronize()
                 assert torch.equal(static_y, eager), (B, S, seed)
         del graph
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_forward_replays_from_a_hip_graph(fp8):
+    """Every entry point enqueues on the caller's stream and neither allocates nor synchronises, so the
+    whole forward (routing, [quantisers,] two GEMMs, merge) can be captured once and replayed.  The
+    replays alternate with eager calls and host synchronisations, and each one is compared with the
+    eager result bit for bit."""
+    from fast_moe_amd.kernels import moe_fp8
+    from fast_moe_amd.kernels.hip import ops
+    T, E, K, D, H = 2048, 16, 2, 256, 384
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(T, D, generator=g)).to(BF16).cuda()
+    v = lambda t: t.permute(0, 2, 1)
+    wg, wu = (v((torch.randn(E, H, D, generator=g) * D ** -0.5).to(BF16).cuda()) for _ in range(2))
+    wd = v((torch.randn(E, D, H, generator=g) * H ** -0.5).to(BF16).cuda())
+    scores = torch.softmax(torch.randn(T, E, generator=g), dim=1).cuda()
+    if fp8:
+        (qg, sg), (qu, su), (qd, sd) = (moe_fp8.quantize_expert_weights(w) for w in (wg, wu, wd))
+
+    def forward():
+        r = ops.route_topk(scores, K)
+        kw = dict(total_rows=T * K)
+        if fp8:
+            qx, sx = ops.quant_rows_fp8(x)
+            hid = ops.grouped_gemm(r["offsets"], qx, qg, row_index=r["gate_index"], index_div=K, b2=qu, epilogue=2,
+                                   a_scale=sx, b_scale=sg, b2_scale=su, **kw)
+            qh, sh = ops.quant_rows_fp8(hid)
+            rows = ops.grouped_gemm(r["offsets"], qh, qd, a_scale=sh, b_scale=sd, **kw)
+        else:
+            hid = ops.grouped_gemm(r["offsets"], x, wg, row_index=r["gate_index"], index_div=K, b2=wu, epilogue=2, **kw)
+            rows = ops.grouped_gemm(r["offsets"], hid, wd, **kw)
+        return ops.combine(rows, r["reverse_index"], r["gates"].to(BF16), r["gate_index"])
+
+    with torch.no_grad():
+        ref = forward().clone()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = forward()
+        torch.cuda.synchronize()
+        for i in range(4):
+            y.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, ref), f"replay {i}"
+            assert torch.equal(forward(), ref)      # eager work between the replays
+            torch.cuda.synchronize()
