@@ -1262,19 +1262,21 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         total_m = s_tab[p.E];
         r_end[0] = 0;
     }
-    // The tiles of an XCD, numbered 0 .. xcd_count-1.  Without a contraction window: one
-    // contiguous range of the tile order (neighbouring tiles share operands in the XCD's L2).
-    // With one the cost of a tile follows its expert's row count, so whole groups are dealt to
-    // the XCDs instead, back and forth (0..7, 7..0, ...): a contiguous range would hand one XCD
-    // all the long experts, and a plain round robin still favours the low XCDs when the experts
-    // come sorted by load.
+    // The tiles of an XCD, numbered 0 .. xcd_count-1.  Paired ring: whole groups (kGroupM row
+    // tiles x all column tiles: what shares operands in an XCD's L2) are dealt to the XCDs back
+    // and forth (0..7, 7..0, ...).  A tile's cost follows its expert (the contraction window of
+    // a weight gradient; a last row tile with few rows runs the shortened main loop), and a
+    // contiguous range per XCD hands one of them all the long experts and another all the short
+    // ones; a plain round robin still favours the low XCDs when the experts come sorted by
+    // load.  4-slot ring: one contiguous range of the tile order per XCD.
     const int64_t total_tiles = (int64_t)total_m * p.n_tiles;
     const int nslots = gridDim.x / kNumXcd;
     const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
     const int64_t group_span = (int64_t)kGroupM * p.n_tiles;
     constexpr bool windowed = KWIN;
+    constexpr bool deal_groups = PAIR;
     int64_t xcd_begin, xcd_count;
-    if (windowed) {
+    if (deal_groups) {
         const int64_t n_groups = (total_m + kGroupM - 1) / kGroupM;
         // rounds of 8 groups; in odd rounds XCD x takes position 7 - x
         const int64_t full_rounds = n_groups / kNumXcd, rest = n_groups % kNumXcd;
@@ -1299,7 +1301,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         else return v / group_span;
     };
     auto to_logical = [&](int64_t j) -> int64_t {
-        if (!windowed) return xcd_begin + j;
+        if (!deal_groups) return xcd_begin + j;
         const int64_t round = div_span(j);
         const int pos = (round & 1) ? kNumXcd - 1 - xcd : xcd;
         return (round * kNumXcd + pos) * group_span + (j - round * group_span);
@@ -2124,7 +2126,8 @@ int launch_ring_cfg(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
     if (TL::PAIR) {
-        if ((p.total_rows / TL::BM + p.E + kGroupM) * (int64_t)p.n_tiles >= ((int64_t)1 << 31))
+        // (tile numbers run up to the row tiles rounded up to a round of kNumXcd groups)
+        if ((p.total_rows / TL::BM + p.E + (kNumXcd + 1) * kGroupM) * (int64_t)p.n_tiles >= ((int64_t)1 << 31))
             return fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: more than 2^31 output tiles");
         magic_u31((int64_t)kGroupM * p.n_tiles, &p.group_magic, &p.group_magic_shift);
     }
