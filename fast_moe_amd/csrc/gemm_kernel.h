@@ -74,6 +74,8 @@ struct GemmParams {
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
     int scale_vec;                      // e4m3: 16-byte loads of 4 weight scales are legal
     int gate_vec;                       // GATED: 8-byte loads of 4 gate values are legal
+    int short_tile_rows;                // paired ring: tiles with at most this many valid rows run the shortened
+                                        // main loop (BM / 2, or 0: never)
     const int64_t* k_window;            // [E+1] per-expert contraction range, or null
     int k_window_multiple;              // every window is a multiple of this and at least twice it (0: unknown)
     uint16_t* aux;                      // SWIGLU: the two pre-activations, or null
@@ -1883,7 +1885,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 barrier();
             }
             load_block(wfa, xfa, cslot, 0, 0, std::true_type{}, std::integral_constant<int, FM>{});
-            const bool sparse = SPARSE && cur.rows_valid <= BM / 2;
+            const bool sparse = SPARSE && cur.rows_valid <= p.short_tile_rows;
             if (wave < NW / 2) {
                 if (sparse) tile_steps(std::integral_constant<int, 0>{}, std::integral_constant<int, SPARSE ? ACT_SPARSE : FM>{});
                 else tile_steps(std::integral_constant<int, 0>{}, std::integral_constant<int, FM>{});
@@ -2011,7 +2013,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 barrier();
             }
             load_w_x0(qwa, qx0, cslot);
-            const bool sparse = SPARSE && cur.rows_valid <= BM / 2;
+            const bool sparse = SPARSE && cur.rows_valid <= p.short_tile_rows;
             if (wave < NW / 2) {
                 if (sparse) tile_steps(std::integral_constant<int, 0>{}, std::integral_constant<bool, SPARSE>{});
                 else tile_steps(std::integral_constant<int, 0>{}, std::false_type{});
@@ -2130,6 +2132,12 @@ int launch_ring_cfg(GemmParams p, hipStream_t stream) {
         if ((p.total_rows / TL::BM + p.E + (kNumXcd + 1) * kGroupM) * (int64_t)p.n_tiles >= ((int64_t)1 << 31))
             return fail(FMOE_ERR_UNSUPPORTED, "fmoe_grouped_gemm: more than 2^31 output tiles");
         magic_u31((int64_t)kGroupM * p.n_tiles, &p.group_magic, &p.group_magic_shift);
+        // A tile that runs the shortened main loop gets ahead of the tiles of its group, which read
+        // the same weights, by about 0.2 us per K-slice; a line lives about 10 us in an XCD's L2.
+        // Up to 64 slices the group keeps sharing its fills and the shortened loop pays (forward
+        // GEMMs of 64 experts -0.6 %, e4m3 at 128 experts -2.4 %); with 128 slices (K = 4096 in bf16,
+        // 2048 rows per expert) the fills it breaks cost more than it saves (GEMM1 +1.8 %).
+        p.short_tile_rows = p.K / (FP8 ? 64 : 32) <= 64 ? TL::BM / 2 : 0;
     }
     auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN, XTR>;
     static bool attr_done = false;
