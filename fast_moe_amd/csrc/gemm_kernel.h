@@ -74,6 +74,7 @@ struct GemmParams {
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
     int scale_vec;                      // e4m3: 16-byte loads of 4 weight scales are legal
     int gate_vec;                       // GATED: 8-byte loads of 4 gate values are legal
+    int gate_vec16;                     // GATED: 16-byte loads of 8 gate values are legal
     int short_tile_rows;                // paired ring: tiles with at most this many valid rows run the shortened
                                         // main loop (BM / 2, or 0: never)
     const int64_t* k_window;            // [E+1] per-expert contraction range, or null
@@ -361,7 +362,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     auto run = [&](auto has_bias_c, auto has_aux_c) {
         constexpr bool HAS_BIAS = decltype(has_bias_c)::value;
         constexpr bool HAS_AUX = SWIGLU && decltype(has_aux_c)::value;   // keep the pre-activations (training)
-        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && !GATED && FN_OUT == 2;   // plain and SiLU epilogues of the ring kernel, bf16 and e4m3
+        constexpr bool QUAD = ALWAYS_VEC && !SWIGLU && FN_OUT == 2;   // plain and SiLU epilogues of the ring kernel, bf16 and e4m3
         // per-column biases of this lane, indexed like rsw
         float bv[FN_OUT][2][2][4], bv2[FN_OUT][2][2][4];
         // with a bias, at least one of the two pointers is set: both loads go through a valid
@@ -391,11 +392,41 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     }
         __builtin_amdgcn_sched_barrier(0);
         FMOE_EPI_STAMP(0);
+        // GATED in the rearranged form: a lane's gate values are the 16 bytes at the position its
+        // store i of a row block writes; the four loads of block fm + 1 go out before block fm's
+        // arithmetic, so that one memory latency per tile is waited for, not one per block.
+        u32x4 gate_next[4] = {};
+        auto fetch_gate = [&](int fm, u32x4 (&g)[4]) {
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            const int quad_row = 4 * ((l & 31) >> 2);
+            const int col = col0 + 32 * (l >> 5) + 8 * (l & 3);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool ok = frag_row(fm) + quad_row + i < rows_valid && col + 7 < p.N;
+                const uint16_t* src = p.aux + (row0 + (ok ? frag_row(fm) + quad_row + i : 0)) * p.aux_stride + (ok ? col : 0);
+                if (p.gate_vec16) {
+                    g[i] = *reinterpret_cast<const u32x4*>(src);
+                } else {
+                    uint32_t e[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) e[j] = ok ? (uint32_t)src[j] : 0u;
+                    g[i] = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
+                }
+            }
+        };
+        if constexpr (QUAD && GATED) fetch_gate(0, gate_next);
         // rows outermost: the stores that complete a row's 128-byte line follow each other
 #pragma unroll
         for (int fm = 0; fm < FM; ++fm) {
             if (fm > 0) FMOE_EPI_STAMP(fm);
             if constexpr (QUAD) {
+                u32x4 gate_cur[4];
+                if constexpr (GATED) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) gate_cur[i] = gate_next[i];
+                    if (fm + 1 < FM) fetch_gate(fm + 1, gate_next);
+                }
                 // The store unit merges what ADJACENT lanes write: a lane and its partner 32 lanes
                 // away cost two requests even for neighbouring bytes, four adjacent lanes on 64
                 // contiguous bytes cost one (a 128 KB tile drains in 1.3 us instead of 3.9).  So:
@@ -477,6 +508,18 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                 const int quad_row = 4 * ((l & 31) >> 2);
                 const int col = col0 + 32 * (l >> 5) + 8 * (l & 3);
                 const uint32_t lane_off = ((uint32_t)quad_row * (uint32_t)p.out_stride + (uint32_t)(32 * (l >> 5) + 8 * (l & 3))) * 2u;
+                if constexpr (GATED) {      // ch holds round(acc + bias): times the rounded SiLU of the gate
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            float ga = __uint_as_float(gate_cur[i][d] << 16), gb = __uint_as_float(gate_cur[i][d] & 0xffff0000u);
+                            ga = fast_silu_f32(ga);
+                            gb = fast_silu_f32(gb);
+                            rbf2(ga, gb);
+                            ch[i][d] = pack_bf16(ga * __uint_as_float(ch[i][d] << 16), gb * __uint_as_float(ch[i][d] & 0xffff0000u));
+                        }
+                }
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     uint16_t* base = obase + i * p.out_stride + col0;
