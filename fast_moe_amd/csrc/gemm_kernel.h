@@ -30,8 +30,10 @@
 //   * Scheduling is on the device: the number of row tiles per expert comes from `offsets`
 //     (wavefront prefix scan), so no max_seq_len and no host synchronisation are needed and
 //     skewed or empty experts cost nothing.  Block ids are dealt round-robin to the 8 XCDs by
-//     the hardware; id -> tile is remapped so that each XCD works on a contiguous range of
-//     tiles (groups of 4 row tiles x all column tiles), which keeps shared rows in its L2.
+//     the hardware; id -> tile is remapped so that each XCD works on whole groups of tiles
+//     (4 row tiles x all column tiles, what shares operands), which keeps them in its L2: the
+//     paired ring deals the groups to the XCDs back and forth, the other kernels give every
+//     XCD one contiguous range of the tile order.
 #pragma once
 
 #include "common.h"
