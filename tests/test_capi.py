@@ -75,6 +75,16 @@ def test_gemm_desc_layout_matches_header():
     assert [int(v) for v in out[1:]] == [getattr(GemmDesc, f).offset for f in fields]
 
 
+def test_enum_values_match_the_header():
+    """The Python constants are the header's enumerators."""
+    from fast_moe_amd.kernels.hip import _lib
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    enums = dict((name, int(value)) for name, value in re.findall(r"\b(FMOE_[A-Z0-9_]+)\s*=\s*(-?\d+)", text))
+    assert (enums["FMOE_EPI_NONE"], enums["FMOE_EPI_SILU"], enums["FMOE_EPI_SWIGLU"], enums["FMOE_EPI_GATED"]) == \
+        (_lib.EPI_NONE, _lib.EPI_SILU, _lib.EPI_SWIGLU, _lib.EPI_GATED)
+    assert (enums["FMOE_F32"], enums["FMOE_BF16"], enums["FMOE_E4M3"]) == (_lib.FMOE_F32, _lib.FMOE_BF16, _lib.FMOE_E4M3)
+
+
 def test_version_and_workspace(lib):
     assert lib.fmoe_version() >= 100
     assert lib.fmoe_route_workspace_bytes(0, 8, 2) > 0
@@ -113,6 +123,26 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
     assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), None) == 1
     assert b"plan is NULL" in lib.fmoe_last_error()
     d.aux = d.aux2 = None
+    # the gated epilogue reads its gate from aux, takes bf16 operands only and no second product
+    d.epilogue = 3
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
+    assert b"GATED reads its gate from aux" in lib.fmoe_last_error()
+    d.aux, d.aux2 = 64, 64
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
+    assert b"aux2 stays NULL" in lib.fmoe_last_error()
+    d.aux2 = None
+    d.aux_stride_row = 4                      # narrower than n
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
+    assert b"aux row stride" in lib.fmoe_last_error()
+    d.aux_stride_row = 8
+    d.a_dtype, d.out_dtype = 0, 0
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 2       # unsupported, not malformed
+    assert b"built for bf16" in lib.fmoe_last_error()
+    d.a_dtype, d.out_dtype = 1, 1
+    d.epilogue = 4
+    assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
+    assert b"unknown epilogue" in lib.fmoe_last_error()
+    d.epilogue, d.aux, d.aux_stride_row = 0, None, 0
     d.a2, d.k2 = 64, 128                     # a second product needs b2 and goes with no epilogue
     assert lib.fmoe_grouped_gemm_plan(ctypes.byref(d), ctypes.byref(plan)) == 1
     assert b"a2 needs b2" in lib.fmoe_last_error()
