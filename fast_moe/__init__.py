@@ -2,19 +2,32 @@
 ``fast_moe.kernels.utils``, ``fast_moe.modules.fast_moe_module``, ``fast_moe.utils.utils`` and
 ``fast_moe.utils.configs`` resolve to the modules of ``fast_moe_amd`` (the same module objects, no
 second copy), so that code written against meta-recsys/fast_moe's operator path imports
-unchanged.  Nothing else of the reference's package is provided here.
+unchanged.  ``fast_moe.dev_settings`` is there as well, and ``fast_moe.kernels.triton.triton_moe``
+names the two option dataclasses the reference's callers import from it (the HIP operators accept
+and ignore them).  Nothing else of the reference's package is provided here.
 """
 import importlib
 import sys
+import types
 
 import fast_moe_amd
 from fast_moe_amd import FastMoELayer, GatingNetwork, KernelType, __version__
 
 for _name in ("kernels", "kernels.utils", "kernels.moe", "kernels.moe_fp8", "modules", "modules.fast_moe_module",
-              "utils", "utils.utils", "utils.configs"):
+              "utils", "utils.utils", "utils.configs", "dev_settings"):
     _mod = importlib.import_module("fast_moe_amd." + _name)
     sys.modules[__name__ + "." + _name] = _mod
     if "." not in _name:
         globals()[_name] = _mod
+
+# the option types under the module path the reference's tests import them from
+_triton = types.ModuleType(__name__ + ".kernels.triton")
+_triton_moe = types.ModuleType(__name__ + ".kernels.triton.triton_moe")
+_triton_moe.__doc__ = "Option dataclasses of the operator API (defined in fast_moe_amd.kernels.moe); no Triton here."
+_triton_moe.IndexSelectJaggedBmmOption = kernels.moe.IndexSelectJaggedBmmOption
+_triton_moe.SiluJaggedBmmCombineOption = kernels.moe.SiluJaggedBmmCombineOption
+_triton.triton_moe = _triton_moe
+sys.modules[_triton.__name__] = _triton
+sys.modules[_triton_moe.__name__] = _triton_moe
 
 __all__ = ["FastMoELayer", "GatingNetwork", "KernelType", "__version__"]

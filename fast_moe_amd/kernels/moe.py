@@ -6,10 +6,9 @@ of /root/reference/kernels/moe.py:39-292.  Differences, all on purpose:
 * ``kernel`` defaults to ``KernelType.HIP`` (the reference defaults to its
   PyTorch path, which this package does not contain); ``KernelType.TRITON`` is
   accepted and runs the same HIP kernels; any other value raises.
-* backward is implemented for index_select_jagged_bmm, index_select_jagged_bmm_swiglu,
-  mul_merge_k_add and silu_jagged_bmm_combine (kernels/hip/autograd.py); the 3D and
-  two-input gating variants and the fp8 operators are forward only and raise when an
-  input requires grad under grad mode.
+* every operator here has a backward (kernels/hip/autograd.py), the 3D and the two-input
+  gating variants included; of the fp8 operators, silu_jagged_bmm_fp8 and silu_jagged_fp8 are
+  forward only (as in the reference) and raise when an input requires grad under grad mode.
 * ``max_seq_len`` is accepted and ignored: tile scheduling reads ``offsets`` on
   the device, so no host synchronisation is needed to obtain it.
 * operands must be bf16 or fp32 CUDA tensors (fp32 runs true-fp32 MFMA, no tf32).

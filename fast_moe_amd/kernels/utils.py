@@ -22,6 +22,25 @@ class KernelType(Enum):
     HIP = "HIP"
 
 
+def _probe_gpu_unavailable():
+    """(skip?, reason) in the form ``unittest.skipIf(*gpu_unavailable)`` takes, as the reference's
+    tests use it (kernels/utils.py:20-25; there: no CUDA device, or a ROCm build).  Here a test can
+    run when a ROCm device is visible and the HIP library has been built."""
+    import os
+
+    from .hip._lib import LIB_PATH
+    if not torch.cuda.is_available() or torch.cuda.device_count() == 0:
+        return True, "no GPU is visible"
+    if not torch.version.hip:
+        return True, "fast_moe_amd runs on ROCm devices (gfx950) only"
+    if not os.path.exists(LIB_PATH):
+        return True, f"{LIB_PATH} has not been built"
+    return False, "a ROCm GPU and libfastmoe_hip.so are present"
+
+
+gpu_unavailable = _probe_gpu_unavailable()
+
+
 def require_hip_kernel(kernel: "KernelType", op: str) -> None:
     """Every operator funnels its ``kernel`` argument through this check."""
     if kernel in (KernelType.HIP, KernelType.TRITON):

@@ -268,3 +268,40 @@ def test_reference_import_paths_resolve():
     import fast_moe_amd.kernels.moe as real
     assert m1 is real and index_select_jagged_bmm is real.index_select_jagged_bmm
     assert K2 is KernelType and L2 is FastMoELayer and callable(bmm_fp8) and callable(_dispatch)
+
+
+def test_imports_of_the_reference_test_files_resolve():
+    """The import block of kernels/tests/moe_test.py:17-28 (and of moe_fp8_test.py, quant_fp8_test.py,
+    test_kernel_parity.py) through the fast_moe.* root."""
+    from fast_moe.dev_settings import get_verbose_level, is_dev_mode, set_dev_mode, set_verbose_level
+    from fast_moe.kernels.triton.triton_moe import IndexSelectJaggedBmmOption, SiluJaggedBmmCombineOption
+    from fast_moe.kernels.utils import (fx_infer_max_len, fx_torch_zeros_like, gpu_unavailable, KernelType,
+                                        to_fp32_if_pytorch_kernel)
+    from fast_moe.modules.fast_moe_module import FastMoELayer
+    from fast_moe.utils.configs import MRNOutput, SGConfig
+    import fast_moe_amd.kernels.moe as real
+    assert IndexSelectJaggedBmmOption is real.IndexSelectJaggedBmmOption
+    assert SiluJaggedBmmCombineOption().activation_checkpointing is False
+    # (skip?, reason), the argument pair of unittest.skipIf
+    skip, reason = gpu_unavailable
+    assert isinstance(reason, str) and reason
+    import torch
+    assert bool(skip) == (not torch.cuda.is_available())
+    import os
+    if "FASTMOE_DEV_MODE" not in os.environ:
+        before = is_dev_mode()
+        set_dev_mode(True)
+        assert is_dev_mode() is True
+        set_dev_mode(before)
+    set_verbose_level(2)
+    assert get_verbose_level() == 2
+    set_verbose_level(0)
+    assert callable(fx_infer_max_len) and callable(fx_torch_zeros_like) and callable(to_fp32_if_pytorch_kernel)
+    assert FastMoELayer and MRNOutput and SGConfig and KernelType.HIP
+
+
+def test_combine_helper_opens_the_reference_profiler_range():
+    """utils/utils.py:55: the merge runs inside record_function("## combine ##")."""
+    import inspect
+    from fast_moe.utils import utils as u
+    assert '"## combine ##"' in inspect.getsource(u._combine)
