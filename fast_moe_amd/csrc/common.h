@@ -49,6 +49,22 @@ __device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
+// round(silu(x)) to bf16 for a bf16-valued x, equal on every one of the 65536 inputs to what
+// x / (1 + exp(-x)) gives when it is evaluated in fp32 with correctly rounded steps and then rounded
+// to bf16 (F.silu on a bf16 tensor).  The fp32 evaluation here may be a few units in the last
+// place off, which only matters when the result lies next to the midpoint of two bf16 values: those
+// (about one input in 4000) are evaluated again in double.  exp(-x) overflows fp32 from x = -88.8
+// down and the quotient is -0 there, as in the fp32 formula; such results never take the second path.
+__device__ __forceinline__ float silu_round_bf16(float x) {
+    float y = x / (1.0f + expf(-x));
+    const uint32_t low = __float_as_uint(y) & 0xffffu;
+    if (low - 0x7ff0u <= 0x20u) {
+        const double xd = (double)x;
+        y = (float)(xd / (1.0 + exp(-xd)));
+    }
+    return round_bf16(y);
+}
+
 // SiLU from the hardware exp / reciprocal (about 2 ulp in fp32): for values that
 // are rounded to bf16 right afterwards.
 __device__ __forceinline__ float fast_silu_f32(float x) {

@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __re
             for (int h = 0; h < 2; ++h) {
                 const float x = bf16_bits_to_f32((va[j] >> (16 * h)) & 0xffffu);
                 const float y = bf16_bits_to_f32((vb[j] >> (16 * h)) & 0xffffu);
-                r |= f32_to_bf16_bits(GATED ? round_bf16(silu_f32(x)) * y : silu_f32(x)) << (16 * h);
+                r |= f32_to_bf16_bits(GATED ? silu_round_bf16(x) * y : silu_round_bf16(x)) << (16 * h);
             }
             vo[j] = r;
         }
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void silu_mul_bf16_kernel(const uint16_t* __re
         for (int64_t i = i0; i < n && i < i0 + 8; ++i) {
             const float x = bf16_bits_to_f32(a[i]);
             const float y = GATED ? bf16_bits_to_f32(b[i]) : 1.0f;
-            out[i] = (uint16_t)f32_to_bf16_bits(GATED ? round_bf16(silu_f32(x)) * y : silu_f32(x));
+            out[i] = (uint16_t)f32_to_bf16_bits(GATED ? silu_round_bf16(x) * y : silu_round_bf16(x));
         }
     }
 }

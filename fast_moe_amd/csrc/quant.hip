@@ -112,8 +112,8 @@ __global__ __launch_bounds__(256) void quant_rows_bf16_wave(
             float lo = bf16_bits_to_f32(v[i][j] & 0xffffu);
             float hi = __uint_as_float(v[i][j] & 0xffff0000u);
             if (SILU) {
-                lo = round_bf16(silu_f32(lo));
-                hi = round_bf16(silu_f32(hi));
+                lo = silu_round_bf16(lo);
+                hi = silu_round_bf16(hi);
                 v[i][j] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
             }
             m = amax_update(m, lo, nan);
@@ -152,8 +152,8 @@ __global__ __launch_bounds__(256) void quant_rows_bf16_block(
         if (SILU) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float lo = round_bf16(silu_f32(bf16_bits_to_f32(v[j] & 0xffffu)));
-                const float hi = round_bf16(silu_f32(__uint_as_float(v[j] & 0xffff0000u)));
+                const float lo = silu_round_bf16(bf16_bits_to_f32(v[j] & 0xffffu));
+                const float hi = silu_round_bf16(__uint_as_float(v[j] & 0xffff0000u));
                 v[j] = (__float_as_uint(lo) >> 16) | (__float_as_uint(hi) & 0xffff0000u);
             }
         }
@@ -195,10 +195,7 @@ __device__ __forceinline__ float load_as_f32<uint16_t>(const uint16_t* p) { retu
 template <typename T, bool SILU>
 __device__ __forceinline__ float fetch(const T* p) {
     float v = load_as_f32<T>(p);
-    if (SILU) {
-        v = silu_f32(v);
-        if (sizeof(T) == 2) v = round_bf16(v);
-    }
+    if (SILU) v = sizeof(T) == 2 ? silu_round_bf16(v) : silu_f32(v);
     return v;
 }
 

@@ -175,3 +175,24 @@ def test_library_cast_path_equals_bit_level_path(dtype):
     q_auto, s_auto = o8.rowwise_quant_fp8(big)
     q_bits, s_bits = o8.rowwise_quant_fp8(big[:64], cast="bits")
     assert torch.equal(q_auto[:64], q_bits) and torch.equal(s_auto[:64], s_bits)
+
+
+def test_silu_bf16_is_torch_silu_on_every_bf16_input():
+    """All 65536 bf16 bit patterns: the oracle's bf16 SiLU against torch's CPU kernel (the library
+    routine the reference calls) and against the fp32 formula with numpy's exp, NaN patterns aside."""
+    import torch
+    from oracle.routing import round_to_bf16
+    bits = (np.arange(65536, dtype=np.uint32) << 16)
+    x = bits.view(np.float32)
+    got = fp8.silu_bf16(x)
+    want = torch.nn.functional.silu(torch.from_numpy(x.copy()).to(torch.bfloat16)).float().numpy()
+    ok = ~np.isnan(want)
+    assert ok.sum() == 65536 - 2 * 127 - 1 and np.all(np.isnan(got[~ok]))      # NaN inputs and -inf
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))
+    with np.errstate(all="ignore"):
+        f32 = round_to_bf16(fp8.silu_f32(x))
+    assert np.array_equal(got[ok].view(np.uint32), f32[ok].view(np.uint32))
+    # closed-form anchors: silu(0) = 0, silu(x) = x beyond 2^5 (x e^-x below half a bf16 step), odd part x / 2
+    assert got[0] == 0 and got[np.uint32(0x4200)] == 32.0            # 0x4200 = 32.0
+    pos, neg = fp8.silu_bf16(np.float32([0.5, 1.0, 3.0])), fp8.silu_bf16(np.float32([-0.5, -1.0, -3.0]))
+    assert np.all(np.abs((pos - neg) - np.float32([0.5, 1.0, 3.0])) <= 2.0 ** -7 * np.float32([0.5, 1.0, 3.0]))
