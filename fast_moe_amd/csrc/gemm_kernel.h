@@ -704,7 +704,15 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
         // inside the caller's steady-state loop, where it would also drain the LDS-DMA stream,
         // which the compiler cannot see, on every iteration.
         FMOE_EPI_STAMP(FM);
-        wait_vmcnt<FM * FN_OUT * 2 * (HAS_AUX ? 3 : 1)>();      // (the scalar-store path issues more)
+        // The number of store instructions issued above, whatever the lanes' predicates: 4 per row
+        // block in the rearranged form, one per column group (and per output tensor) otherwise.
+        // The ring kernel's first double step of the next tile skips its own counted wait on the
+        // strength of this one (see skip_wait there), which is only sound when every one of these
+        // stores was issued unconditionally, i.e. through store16_uniform_base (ALWAYS_VEC).
+        constexpr int kStoresIssued = FM * (QUAD ? 4 : FN_OUT * 2 * (HAS_AUX ? 3 : 1));
+        static_assert(!QUAD || FN_OUT * 2 == 4, "the rearranged form stores as many pieces as the column-group form");
+        static_assert(kStoresIssued <= 63, "vmcnt is a 6-bit field");
+        wait_vmcnt<kStoresIssued>();      // (the scalar-store path issues more)
         after_stores();
     };
     if (SWIGLU && p.aux) {
@@ -1185,6 +1193,10 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
     constexpr int BM = TL::BM, BN = TL::BN, NW = TL::NW, STAGES = TL::STAGES;
     constexpr int FM = TL::FM, FN = TL::FN, TM = TL::TM, TN = TL::TN;
     constexpr bool PAIR = TL::PAIR;
+    // (the epilogue is instantiated with ALWAYS_VEC = true below: its stores go through
+    // store16_uniform_base, are all issued, and end with a counted wait, which the first double
+    // step of the following tile relies on when it skips its own)
+    constexpr bool kEpilogueStoresUnconditional = true;
     constexpr int NR = PAIR ? TL::NREG : 1;
     constexpr int ESIZE = FP8 ? 1 : 2;
     constexpr int BK = 64 / ESIZE;
@@ -2100,7 +2112,8 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane, convert_rows,
             (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2)) ? tstamp + 12 : nullptr);
 #else
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR, ROW_IL>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
+        static_assert(kEpilogueStoresUnconditional, "skip_wait needs an epilogue whose stores are all issued");
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, kEpilogueStoresUnconditional, PAIR, XTR, ROW_IL>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
                                                                 done.rows_valid, wm, wn, lane, convert_rows);
 #endif
 #ifdef FMOE_TRACE

@@ -640,6 +640,15 @@ extern "C" int fmoe_route_topk_static(const void* scores, int score_dtype, int64
     FMOE_REQUIRE(T <= FMOE_ROUTE_STATIC_MAX_POSITIONS && T * (int64_t)K <= FMOE_ROUTE_STATIC_MAX_POSITIONS,
                  "%s: T*K=%lld routed positions exceed the %d the built-in scratch holds (use fmoe_route_topk "
                  "with a workspace)", who, (long long)T * K, FMOE_ROUTE_STATIC_MAX_POSITIONS);
+    // every check that can refuse the call comes before the scratch lookup, so that a refused call
+    // never touches the runtime (the first lookup on a device calls hipGetSymbolAddress)
+    FMOE_REQUIRE(K <= 64 && K <= E, "%s: K=%d must be at most 64 and at most E=%d", who, K, E);
+    FMOE_REQUIRE(renorm >= 0 && renorm <= 3, "%s: gate mode %d is not one of 0..3", who, renorm);
+    FMOE_REQUIRE(score_dtype == FMOE_F32 || score_dtype == FMOE_BF16, "%s: scores must be fp32 or bf16", who);
+    FMOE_REQUIRE(lengths && offsets, "%s: lengths/offsets are NULL", who);
+    if (T > 0)
+        FMOE_REQUIRE(scores && topk_idx && gates && gate_index && token_index && reverse_index,
+                     "%s: NULL tensor pointer", who);
     if (make_plan(T, E, K).total_bytes > kStaticScratchBytes)
         return fail(FMOE_ERR_WORKSPACE, "%s: the call needs %zu B of scratch, the built-in buffer has %zu B", who,
                     make_plan(T, E, K).total_bytes, kStaticScratchBytes);

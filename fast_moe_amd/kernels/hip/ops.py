@@ -86,9 +86,18 @@ def route_topk(scores: torch.Tensor, k: int, renorm=True, static_scratch: bool =
             "token_index": torch.empty((T * k,), **i64),
             "reverse_index": torch.empty((T, k), **i64),
         }
-    elif (tuple(out["topk_idx"].shape) != (T, k) or out["gates"].dtype != scores.dtype
-          or out["lengths"].numel() != E or out["gate_index"].device != dev):
-        raise ValueError("route_topk: `out` was made for other shapes")
+    else:
+        # the kernels write every one of these through raw pointers: shape, dtype, device and
+        # contiguity of each are checked, not only of the first few
+        want = {"topk_idx": ((T, k), torch.int64), "gates": ((T, k), scores.dtype), "lengths": ((E,), torch.int64),
+                "offsets": ((E + 1,), torch.int64), "gate_index": ((T * k,), torch.int64),
+                "token_index": ((T * k,), torch.int64), "reverse_index": ((T, k), torch.int64)}
+        for name, (shape, dtype) in want.items():
+            t = out.get(name)
+            if (t is None or tuple(t.shape) != shape or t.dtype != dtype or t.device != dev
+                    or not t.is_contiguous()):
+                raise ValueError(f"route_topk: out[{name!r}] must be a contiguous {dtype} tensor of shape {shape} on "
+                                 f"{dev} (a dict of a previous call with the same T, E, k and score dtype)")
     lib = _lib.load()
     if static_scratch:
         rc = lib.fmoe_route_topk_static(

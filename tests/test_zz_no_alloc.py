@@ -59,10 +59,13 @@ def test_static_scratch_routing_equals_workspace_routing_on_consecutive_calls():
         scores = scores_of(T, E, 40 + n, dtype)
         want, got = outputs(T, E, K, dtype), outputs(T, E, K, dtype)
         assert call_workspace(lib, scores, K, renorm, want) == 0, lib.fmoe_last_error()
-        before = torch.cuda.memory_allocated()
-        assert call_static(lib, scores, K, renorm, got) == 0, lib.fmoe_last_error()
-        assert torch.cuda.memory_allocated() == before          # (torch's view; the library has no allocator call)
         torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+        assert call_static(lib, scores, K, renorm, got) == 0, lib.fmoe_last_error()
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == before          # torch's allocator saw nothing ...
+        if n > 0:       # ... and the device's free memory did not move either (hipMemGetInfo sees a
+            assert torch.cuda.mem_get_info()[0] == free_before  # hipMalloc inside the library; call 0 loads code objects)
         for key in KEYS:
             a, b = got[key], want[key]
             if a.dtype != torch.int64:
@@ -87,6 +90,48 @@ def test_static_scratch_routing_through_the_wrapper_and_empty_input():
     assert empty["offsets"].cpu().tolist() == [0] * 9
 
 
+def test_static_scratch_routing_replays_from_a_captured_graph():
+    """The use the entry point is for: captured into a HIP graph (after one call outside the capture,
+    which looks the scratch address up), replayed with new scores in the same buffers, every replay
+    bit-identical to the eager workspace routing of those scores."""
+    from fast_moe_amd.kernels.hip import ops
+    T, E, K = 2048, 64, 8
+    scores = scores_of(T, E, 11, torch.float32)
+    out = ops.route_topk(scores, K, static_scratch=True)             # outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.route_topk(scores, K, static_scratch=True, out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (12, 13, 14):
+        scores.copy_(scores_of(T, E, seed, torch.float32))
+        want = ops.route_topk(scores, K)                                 # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for key in KEYS:
+            assert torch.equal(out[key], want[key]), (key, seed)
+
+
+def test_route_topk_checks_every_tensor_of_out():
+    from fast_moe_amd.kernels.hip import ops
+    scores = scores_of(128, 16, 3, torch.float32)
+    good = ops.route_topk(scores, 4)
+    for name, bad in (("offsets", good["offsets"][:-1]), ("gate_index", good["gate_index"].to(torch.int32)),
+                      ("token_index", good["token_index"][: 128 * 4 - 1]),
+                      ("reverse_index", good["reverse_index"].t().contiguous().t()),
+                      ("gates", good["gates"].to(torch.bfloat16)), ("lengths", good["lengths"].cpu())):
+        out = dict(good)
+        out[name] = bad
+        with pytest.raises(ValueError, match=name):
+            ops.route_topk(scores, 4, out=out)
+    with pytest.raises(ValueError, match="topk_idx"):
+        ops.route_topk(scores, 4, out={k: v for k, v in good.items() if k != "topk_idx"})
+
+
 def test_static_scratch_routing_turns_away_what_does_not_fit():
     from fast_moe_amd.kernels.hip import _lib
     lib = _lib.load()
@@ -99,3 +144,10 @@ def test_static_scratch_routing_turns_away_what_does_not_fit():
     scores = scores_of(4, 600, 1, torch.float32)
     out = outputs(4, 600, 2, torch.float32)
     assert call_static(lib, scores, 2, 1, out) == 1 and b"experts" in lib.fmoe_last_error()
+    # K beyond E or 64 and an unknown gate mode are refused by the entry point's own checks
+    scores = scores_of(16, 8, 1, torch.float32)
+    out = outputs(16, 8, 9, torch.float32)
+    assert call_static(lib, scores, 9, 1, out) == 1 and b"K=9" in lib.fmoe_last_error()
+    out = outputs(16, 8, 2, torch.float32)
+    assert call_static(lib, scores, 2, 7, out) == 1 and b"gate mode" in lib.fmoe_last_error()
+    assert int(out["offsets"][0]) == -1
