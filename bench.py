@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_bf16|c4_fp8|c2_bf16|c5_bf16|c5_fp8]
                     [--tokens T] [--no-cpu-baseline] [--no-extra] [--sample-clock] [--dense-reference]
+                    [--hbm-ceiling]
 
 A step is one forward pass of the hot path over one batch of synthetic input that is
 already resident in HBM: top-k routing from the gate probabilities, the gather +
@@ -156,7 +157,7 @@ class GpuPath:
                                          row_index=r["gate_index"], index_div=K, bias=self.inp["b1"], epilogue=1)
         elif self.fp8:
             self.hidden = o.grouped_gemm(r["offsets"], self.qx, self.qg, total_rows=R, row_index=r["gate_index"],
-                                         index_div=K, b2=self.qu, epilogue=2, a_scale=self.sx, b_scale=self.sg,
+                                         index_div=K, b2=self.qu, epilogue=2, scales_pow2=True, a_scale=self.sx, b_scale=self.sg,
                                          b2_scale=self.su)
         else:
             self.hidden = o.grouped_gemm(r["offsets"], self.inp["x"], self.wg, total_rows=R,
@@ -171,7 +172,7 @@ class GpuPath:
         if self.w["kind"] == "mlp":
             self.rows = o.grouped_gemm(r["offsets"], self.hidden, self.w2, total_rows=R, bias=self.inp["b2"])
         elif self.fp8:
-            self.rows = o.grouped_gemm(r["offsets"], self.qh, self.qd, total_rows=R, a_scale=self.sh,
+            self.rows = o.grouped_gemm(r["offsets"], self.qh, self.qd, total_rows=R, scales_pow2=True, a_scale=self.sh,
                                        b_scale=self.sd)
         else:
             self.rows = o.grouped_gemm(r["offsets"], self.hidden, self.wd, total_rows=R)
@@ -545,6 +546,46 @@ def sustained(fn, seconds, sampler_period=0.25):
     return ms, clock
 
 
+def hbm_ceiling(gib=4, reps=20):
+    """GB/s of kernels that do nothing but memory accesses over `gib` GiB (far beyond the 256 MB
+    last-level cache): the library's probe kernel (16-byte accesses, eight in flight per lane, at
+    two grid sizes) and torch's own reduction, fill and copy.  The fraction-of-HBM figures of the
+    quantisers and of the merge are to be read against these, not only against the 8 TB/s of the
+    data sheet."""
+    from fast_moe_amd.kernels.hip import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    nbytes = gib << 30
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    buf.view(torch.int32).random_(0, 1 << 20)
+    stream = torch.cuda.current_stream(dev)
+    out = {"bytes": nbytes, "launches": reps}
+
+    def probe(mode, blocks):
+        _lib.check(lib.fmoe_hbm_probe(buf.data_ptr(), nbytes, mode, blocks, stream.cuda_stream), "fmoe_hbm_probe")
+
+    for name, mode, moved in (("read", 0, nbytes), ("write", 1, nbytes), ("copy", 2, nbytes)):
+        for blocks in (2048, 32768):
+            fn = lambda: probe(mode, blocks)
+            fn()
+            torch.cuda.synchronize()
+            ms = time_region(fn, reps, stream)
+            out[f"probe_{name}_{blocks}_blocks"] = {"ms": round(ms, 4), "gbs": round(moved / ms / 1e6, 1),
+                                                    "frac_hbm": round(moved / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    as_f32, half = buf.view(torch.float32), nbytes // 2
+    for name, fn, moved in (("torch_sum_fp32", lambda: as_f32.sum(), nbytes),
+                            ("torch_fill", lambda: buf.fill_(1), nbytes),
+                            ("torch_copy", lambda: buf[half:].copy_(buf[:half]), nbytes)):
+        fn()
+        torch.cuda.synchronize()
+        ms = time_region(fn, reps, stream)
+        out[name] = {"ms": round(ms, 4), "gbs": round(moved / ms / 1e6, 1),
+                     "frac_hbm": round(moved / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    del buf
+    torch.cuda.empty_cache()
+    return out
+
+
 def sustained_section(w, sample_clock, dense_reference, seconds=3.0):
     """Each GEMM of the workload run back to back for ~3 s: milliseconds per launch, TFLOP/s, and the
     shader clock rocm-smi reports meanwhile; with `dense_reference` the vendor's dense GEMM
@@ -563,6 +604,29 @@ def sustained_section(w, sample_clock, dense_reference, seconds=3.0):
         if clock:
             entry["frac_of_peak_at_clock"] = round(fl / ms / 1e9 / (peak * clock["median_mhz"] / 2400.0), 4)
         out[name] = entry
+    if dense_reference and w["dtype"] == "fp8":
+        # the vendor's e4m3 GEMM with row-wise scales (torch._scaled_mm -> hipBLASLt), one product of
+        # the same FLOPs per GEMM of the workload, operands quantised by the library's own quantiser
+        from fast_moe_amd.kernels.hip import ops
+        R = w["T"] * w["K"]
+        hn = 2 * w["H"] if w["kind"] == "swiglu" else w["H"]
+        for name, (m, k, n) in (("dense_gemm1", (R, w["D"], hn)), ("dense_gemm2", (R, w["H"], w["O"]))):
+            try:
+                qa, sa = ops.quant_rows_fp8(torch.randn(m, k, device=dev).to(torch.bfloat16))
+                qb, sb = ops.quant_rows_fp8((torch.randn(n, k, device=dev) * k ** -0.5).to(torch.bfloat16))
+                ra, rb = (1.0 / sa).view(m, 1).contiguous(), (1.0 / sb).view(1, n).contiguous()
+                fn = lambda: torch._scaled_mm(qa, qb.t(), scale_a=ra, scale_b=rb, out_dtype=torch.bfloat16)
+                fn()
+                torch.cuda.synchronize()
+                ms, clock = sustained(fn, seconds)
+                fl = 2.0 * m * k * n
+                entry = {"kernel": "torch._scaled_mm, e4m3fn x e4m3fn, row-wise fp32 scales, bf16 out",
+                         "shape_mkn": [m, k, n], "ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "sclk": clock}
+                if clock:
+                    entry["frac_of_peak_at_clock"] = round(fl / ms / 1e9 / (PEAK["fp8"] * clock["median_mhz"] / 2400.0), 4)
+            except Exception as exc:        # not every hipBLASLt build has the row-wise form
+                entry = {"shape_mkn": [m, k, n], "unavailable": f"{type(exc).__name__}: {exc}"[:300]}
+            out[name] = entry
     if dense_reference and w["dtype"] == "bf16":
         R = w["T"] * w["K"]
         hn = 2 * w["H"] if w["kind"] == "swiglu" else w["H"]
@@ -591,8 +655,10 @@ def with_wq(entry, timing, flops):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # (100 steps: the K-step figure then agrees with the per-step HIP-event median; with 20, the one
+    # pipeline fill after the synchronisation and the final synchronisation weigh 2.5 % of the step)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3_bf16", choices=sorted(WORKLOADS))
     ap.add_argument("--tokens", type=int, default=None, help="override the token count (C5 sweep)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -607,6 +673,9 @@ def main():
     ap.add_argument("--dense-reference", action="store_true",
                     help="also time the vendor's dense GEMM (torch.matmul) on the FLOP-equivalent single product "
                          "of each GEMM of the workload, with the shader clock, for scale")
+    ap.add_argument("--hbm-ceiling", action="store_true",
+                    help="also stream 4 GiB with kernels that only read, only write, and copy (fmoe_hbm_probe, and "
+                         "torch's sum / fill_ / copy_ beside them): what the part gives a memory-bound kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 512 MiB device copy, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -686,6 +755,8 @@ def main():
             line["extra"].update(extra_workloads(args.steps, args.warmup))
     if args.sample_clock or args.dense_reference:
         line["sustained"] = sustained_section(w, args.sample_clock, args.dense_reference)
+    if args.hbm_ceiling:
+        line["hbm_ceiling"] = hbm_ceiling()
     if args.calibrate_copy:      # a kernel of known traffic: 512 MiB read + 512 MiB written
         src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)

@@ -83,10 +83,61 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ sr
     }
 }
 
+// HBM probe: what this part reads and writes per second when nothing else limits a kernel.
+// Blocks of 256 lanes take 32 KB pieces of the buffer round robin; a lane has eight 16-byte
+// accesses in flight.  READ: non-temporal loads folded into a value that is stored only if it
+// takes a value no buffer produces in practice (the loads cannot be dropped).  WRITE: 16-byte
+// stores of a pattern.  COPY: first half of the buffer to the second.
+template <int MODE>
+__global__ __launch_bounds__(256) void hbm_probe_kernel(u32x4* __restrict__ buf, int64_t pieces, uint32_t* sink) {
+    constexpr int PER = 8;                      // 16-byte accesses per lane and piece: 256 * 8 * 16 B = 32 KB
+    u32x4 acc = {0, 0, 0, 0};
+    const int64_t half = pieces * 256 * PER;    // COPY: the second half starts here (in 16-byte units)
+    for (int64_t pc = blockIdx.x; pc < pieces; pc += gridDim.x) {
+        u32x4* base = buf + pc * 256 * PER + threadIdx.x;
+        if (MODE == 0) {
+            u32x4 v[PER];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) v[i] = __builtin_nontemporal_load(base + i * 256);
+#pragma unroll
+            for (int i = 0; i < PER; ++i) acc ^= v[i];
+        } else if (MODE == 1) {
+            const uint32_t x = (uint32_t)pc;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) base[i * 256] = u32x4{x, x + 1, x + 2, x + 3};
+        } else {
+            u32x4 v[PER];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) v[i] = __builtin_nontemporal_load(base + i * 256);
+#pragma unroll
+            for (int i = 0; i < PER; ++i) base[half + i * 256] = v[i];
+        }
+    }
+    if (MODE == 0 && (acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) *sink = acc[0];
+}
+
 }  // namespace
 }  // namespace fmoe
 
 using namespace fmoe;
+
+extern "C" int fmoe_hbm_probe(void* buf, int64_t bytes, int mode, int blocks, fmoe_stream_t stream) {
+    FMOE_REQUIRE(buf && aligned16(buf), "fmoe_hbm_probe: buf must be a 16-byte aligned device pointer");
+    FMOE_REQUIRE(mode >= 0 && mode <= 2, "fmoe_hbm_probe: mode must be 0 (read), 1 (write) or 2 (copy)");
+    const int64_t piece = 256 * 8 * 16;
+    const int64_t span = mode == 2 ? bytes / 2 : bytes;
+    FMOE_REQUIRE(bytes >= 2 * piece && span % piece == 0,
+                 "fmoe_hbm_probe: bytes must be a multiple of %lld (twice that for a copy)", (long long)piece);
+    FMOE_REQUIRE(blocks >= 1 && blocks <= (1 << 20), "fmoe_hbm_probe: 1 .. 2^20 blocks");
+    const int64_t pieces = span / piece;
+    u32x4* b = (u32x4*)buf;
+    uint32_t* sink = (uint32_t*)buf;
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == 0) hbm_probe_kernel<0><<<blocks, 256, 0, s>>>(b, pieces, sink);
+    else if (mode == 1) hbm_probe_kernel<1><<<blocks, 256, 0, s>>>(b, pieces, sink);
+    else hbm_probe_kernel<2><<<blocks, 256, 0, s>>>(b, pieces, sink);
+    return check_launch("fmoe_hbm_probe");
+}
 
 extern "C" int fmoe_transpose_last2(const void* src, void* dst, int elem_size, int64_t batch, int64_t rows,
                                     int64_t cols, int64_t src_stride_b, int64_t src_stride_r,

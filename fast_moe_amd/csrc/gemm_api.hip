@@ -148,6 +148,7 @@ static int prepare_gemm(const fmoe_gemm_desc* d, GemmParams& p, int& sel) {
     p.short_tile_rows = 0;      // (the paired ring's launcher decides)
     p.gate_vec16 = gated && aligned16(d->aux) && d->aux_stride_row % 8 == 0;
     p.gate_vec = gated && (reinterpret_cast<uintptr_t>(d->aux) % 8 == 0) && d->aux_stride_row % 4 == 0;
+    p.scale_pow2 = fp8 && d->scale_pow2 != 0;
     p.scale_vec = fp8 && d->n >= 4 && d->n % 4 == 0 && aligned16(d->b_scale) && (!d->b2_scale || aligned16(d->b2_scale));
     const int esize = fp8 ? 1 : (f32 ? 4 : 2);
     const int chunk = 16 / esize;

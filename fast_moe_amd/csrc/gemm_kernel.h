@@ -75,6 +75,7 @@ struct GemmParams {
     int n_tiles;
     int vec_store;                      // 16-byte stores of 8 bf16 are legal
     int scale_vec;                      // e4m3: 16-byte loads of 4 weight scales are legal
+    int scale_pow2;                     // e4m3: the caller promises that every scale is an exact power of two
     int gate_vec;                       // GATED: 8-byte loads of 4 gate values are legal
     int gate_vec16;                     // GATED: 16-byte loads of 8 gate values are legal
     int short_tile_rows;                // paired ring: tiles with at most this many valid rows run the shortened
@@ -223,10 +224,62 @@ __device__ __forceinline__ void store16_uniform_base(const void* base, uint32_t 
 // nothing).  The ring kernel converts the row indices it fetched before the epilogue there.
 struct NoAfterStores {
     __device__ __forceinline__ void operator()() const {}
+    __device__ __forceinline__ void block_done(int) const {}
 };
+// block_done(fm): called behind the stores of the wave's row block fm (straight-line code as well);
+// the ring kernel issues the next tile's scale loads there, under the arithmetic of the blocks left.
+template <typename BlockDone, typename AfterAll>
+struct EpilogueHooks {
+    BlockDone on_block;
+    AfterAll on_end;
+    __device__ __forceinline__ void operator()() const { on_end(); }
+    __device__ __forceinline__ void block_done(int fm) const { on_block(fm); }
+};
+template <typename BlockDone, typename AfterAll>
+__device__ __forceinline__ EpilogueHooks<BlockDone, AfterAll> make_hooks(BlockDone b, AfterAll a) {
+    return EpilogueHooks<BlockDone, AfterAll>{b, a};
+}
 
+// E8M0 code (2^(code - 127)) of the reciprocal of a power-of-two fp32 scale: what the scale
+// operands of v_mfma_scale_f32_32x32x64_f8f6f4 take.  2^127 (the quantiser's scale of an all-zero
+// or non-finite row) gives code 0 = 2^-127.
+__device__ __forceinline__ uint32_t e8m0_of_reciprocal(float scale) {
+    return (254u - (__float_as_uint(scale) >> 23)) & 0xffu;
+}
+// one e4m3 MFMA whose products are scaled by 2^(byte OA of sa - 127) per weight row and
+// 2^(byte OB of sb - 127) per activation row (lane l: row l % 32 of its fragment).
+// Written as inline assembly with the accumulator tied to the destination: through the builtin the
+// destination is a separate early-clobber operand, which costs the ring kernel (at 256 registers
+// with 128 of them accumulators) about 50 spilled registers per lane around the tile boundary.
+// The compiler therefore does not know that this is an MFMA and inserts none of the wait states
+// the matrix pipe needs around VALU accesses to its registers.  VALU write -> MFMA read (the
+// clears of a tile's accumulators, the packed scale codes): two idle issue cycles stand in front
+// of every one of these instructions, inside the same statement (they pass while the pipe works
+// on the MFMA before).  MFMA write -> VALU read (the epilogue): mfma_results_guard() behind the
+// main loop.
+template <int OA, int OB>
+__device__ __forceinline__ void mfma_e4m3_scaled(const i32x8& a, const i32x8& b, f32x16& c, uint32_t sa, uint32_t sb) {
+    asm volatile("s_nop 1\n\tv_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+                 : "+v"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb), "n"(OA & 1), "n"(OB & 1), "n"(OA >> 1), "n"(OB >> 1));
+}
+// 32 idle issue cycles behind the last of those MFMAs (a 16-pass MFMA needs 18 before the VALU may
+// read its result), and nothing that follows in the program may be scheduled in front of them.
+__device__ __forceinline__ void mfma_results_guard() {
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// MSC (e4m3): the scales were applied by the MFMAs themselves (power-of-two scales as block scales of
+// the instruction): acc already holds sum / (s_a * s_w) and the epilogue loads and multiplies nothing.
 template <int FM, int FN, int TM, int TN, bool FP8, int EPI, bool ALWAYS_VEC = false, bool ROWS32 = false,
-          bool OUT2 = false, bool ROW_IL = false, typename AfterStores = NoAfterStores>
+          bool OUT2 = false, bool ROW_IL = false, typename AfterStores = NoAfterStores, bool MSC = false>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)[FN][FM], int expert,
                                               int n0, int64_t row0, int rows_valid, int wm, int wn,
                                               int lane, AfterStores after_stores = AfterStores(),
@@ -275,7 +328,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
     // nq + 8*q + 4*khalf + j with nq = first column of register-quad pair gp of fragment fn
     float rsw[FN_OUT][2][2][4], rsw2[FN_OUT][2][2][4];
     const int col0 = n0 + (SWIGLU ? wn * (TN / 2) : wn * TN);
-    if (FP8) {
+    constexpr bool SCALE = FP8 && !MSC;         // divide the scales out here
+    if (SCALE) {
         // the activation scales of this lane's rows: all index loads, then all scale loads (two
         // memory latencies, not two per row block)
         typedef typename std::conditional<ROWS32, int32_t, int64_t>::type row_t;
@@ -447,8 +501,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                 const int v = 4 * (2 * gp + q) + j;
                                 float ya = acc[fn][fm][v], yb = acc[fn][fm][v + 1];
                                 if (FP8) {
-                                    ya *= rsa[fm] * rsw[fn][gp][q][j];
-                                    yb *= rsa[fm] * rsw[fn][gp][q][j + 1];
+                                    if (SCALE) {
+                                        ya *= rsa[fm] * rsw[fn][gp][q][j];
+                                        yb *= rsa[fm] * rsw[fn][gp][q][j + 1];
+                                    }
                                     if (HAS_BIAS && p.bias) {
                                         rbf2(ya, yb);
                                         ya += bv[fn][gp][q][j];
@@ -529,6 +585,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     store16_uniform_base(base, ok ? lane_off : kDropLane, u32x4{ch[i][0], ch[i][1], ch[i][2], ch[i][3]});
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                after_stores.block_done(fm);
                 continue;
             }
             // GATED: the row block's gate values, all loads of the block issued together (one memory
@@ -582,8 +639,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                             float ua = SWIGLU ? acc[fn + FN / 2][fm][v] : 0.0f;
                             float ub = SWIGLU ? acc[fn + FN / 2][fm][v + 1] : 0.0f;
                             if (FP8) {
-                                ya *= rsa[fm] * rsw[fn][gp][q][j];
-                                yb *= rsa[fm] * rsw[fn][gp][q][j + 1];
+                                if (SCALE) {
+                                    ya *= rsa[fm] * rsw[fn][gp][q][j];
+                                    yb *= rsa[fm] * rsw[fn][gp][q][j + 1];
+                                }
                                 rbf2(ya, yb);
                                 if (HAS_BIAS && p.bias) {
                                     ya += bv[fn][gp][q][j];
@@ -591,8 +650,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                                     rbf2(ya, yb);
                                 }
                                 if (SWIGLU) {
-                                    ua *= rsa[fm] * rsw2[fn][gp][q][j];
-                                    ub *= rsa[fm] * rsw2[fn][gp][q][j + 1];
+                                    if (SCALE) {
+                                        ua *= rsa[fm] * rsw2[fn][gp][q][j];
+                                        ub *= rsa[fm] * rsw2[fn][gp][q][j + 1];
+                                    }
                                     rbf2(ua, ub);
                                     if (HAS_BIAS && p.bias2) {
                                         ua += bv2[fn][gp][q][j];
@@ -696,6 +757,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams& p, f32x16 (&acc)
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
+            after_stores.block_done(fm);
         }
         // Everything older than this epilogue's own stores has completed: a wait that costs
         // nothing (the loads it names were needed above) but tells the compiler so.  Without it
@@ -1183,8 +1245,17 @@ __device__ __forceinline__ int uniform_lane(int v, int src_lane) {
 // the fragments are masked beyond the window's end.  The rows read past the end belong to the
 // next expert or, after the last one, to the slack the caller promises (k_slack_rows >= 128
 // readable rows behind both operands; their contents do not matter).
-template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false>
+// MSC (e4m3, paired ring): the row-wise scales are powers of two (p.scale_pow2) and are applied by
+// the MFMAs themselves: every wave keeps the E8M0 codes of the reciprocal scales of its four
+// activation row blocks and its two weight fragments in two registers, which are the block-scale
+// operands of v_mfma_scale_f32_32x32x64_f8f6f4 (a power-of-two factor on all 64 products of an
+// output element in every K-step: the accumulator holds exactly what the division in the epilogue
+// would give).  The scales of the next tile are fetched inside the epilogue of the current one
+// (row indices before it, the scales behind its first row block, packed at its end), so that no
+// tile waits for an index -> scale chain and the epilogue multiplies nothing.
+template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false, bool MSC = false>
 __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmParams p) {
+    static_assert(!MSC || (FP8 && TL::PAIR && !KWIN && !WTR && !XTR), "MFMA-applied scales: e4m3 on the paired ring");
     static_assert(!WTR || (TL::PAIR && !FP8 && TL::BN == 256 && TL::NW == 8),
                   "in-place N-contiguous weights: bf16, paired ring, 256-column tiles of 8 waves");
     static_assert(!KWIN || TL::PAIR, "contraction windows: paired ring");
@@ -1619,6 +1690,57 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         xtr_off[fm] = (frag0 / (BM / 2)) * 8192 + row * 256 + (((ncol >> 3) ^ (4 * (l16 >> 2))) << 4) + (ncol & 7) * 2;
     }
 
+    // MSC: E8M0 codes of this lane's reciprocal scales, byte fm of sc_x for activation row block fm
+    // (row lane & 31 of it), byte fn of sc_w for weight fragment fn (its column lane & 31)
+    uint32_t sc_x = 0x7f7f7f7fu, sc_w = 0x7f7f7f7fu;
+    // (sc_idx: row_index entries (low halves) of the lane's rows, or the rows themselves)
+    auto sc_fetch_rows = [&](const TileInfo& t, int32_t (&sc_idx)[FM]) {       // hop 1: which source rows
+        if constexpr (MSC) {
+            int l = lane;
+            asm volatile("" : "+v"(l));
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) {
+                const int tr = (ROW_IL ? (fm * 2 + wm) * 32 : wm * TM + fm * 32) + (l & 31);
+                const int32_t r = (int32_t)t.row0 + (tr < t.rows_valid ? tr : 0);
+                sc_idx[fm] = p.row_index ? reinterpret_cast<const int32_t*>(p.row_index)[2 * (int64_t)r] : r;
+            }
+        }
+    };
+    auto sc_fetch_scales = [&](const TileInfo& t, const int32_t (&sc_idx)[FM], float (&sc_xraw)[FM], float (&sc_wraw)[FN]) {     // hop 2: the scales themselves
+        if constexpr (MSC) {
+            int l = lane;
+            asm volatile("" : "+v"(l));
+            const int32_t last = (int32_t)(p.a_rows - 1);
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) {
+                int32_t src = p.row_index ? div_index32(p, sc_idx[fm]) : sc_idx[fm];
+                src = src < 0 ? 0 : (src > last ? last : src);
+                sc_xraw[fm] = p.a_scale[src];
+            }
+            const int expert = __builtin_amdgcn_readfirstlane(t.expert);
+            const int n0 = t.nt * BN_OUT;
+#pragma unroll
+            for (int fn = 0; fn < FN; ++fn) {
+                const bool up = SWIGLU && fn >= FN / 2;
+                int n = n0 + (SWIGLU ? wn * (TN / 2) + (fn % (FN / 2)) * 32 : wn * TN + fn * 32) + (l & 31);
+                n = n < p.N ? n : p.N - 1;
+                sc_wraw[fn] = (up ? p.b2_scale : p.b_scale)[(int64_t)expert * p.N + n];
+            }
+        }
+    };
+    auto sc_pack = [&](const float (&sc_xraw)[FM], const float (&sc_wraw)[FN]) {
+        if constexpr (MSC) {
+            uint32_t x = 0, w = 0x7f7f7f7fu;
+#pragma unroll
+            for (int fm = 0; fm < FM; ++fm) x |= e8m0_of_reciprocal(sc_xraw[fm]) << (8 * fm);
+            static_assert(FM == 4 && FN <= 4, "one byte per row block / weight fragment");
+#pragma unroll
+            for (int fn = 0; fn < FN; ++fn) w = (w & ~(0xffu << (8 * fn))) | (e8m0_of_reciprocal(sc_wraw[fn]) << (8 * fn));
+            sc_x = x;
+            sc_w = w;
+        }
+    };
+
     if (slot >= xcd_count) return;
     const int my_tiles = (int)((xcd_count - slot + nslots - 1) / nslots);
     // 4-slot ring: every item of the block; paired ring: issue_next only starts the first tile
@@ -1653,6 +1775,13 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
         fetch_rows(cur, r0);
         rows_to_offsets(r0, x0);
         make_ptrs(cur, x0);
+    }
+    if constexpr (MSC) {                    // the first tile's scales: fetched here, in the open
+        int32_t idx0[FM];
+        float xraw0[FM], wraw0[FN];
+        sc_fetch_rows(cur, idx0);
+        sc_fetch_scales(cur, idx0, xraw0, wraw0);
+        sc_pack(xraw0, wraw0);
     }
     auto enter_next = [&]() {               // the issue side moves on to the next tile
         make_ptrs(nxt, xoff_next);
@@ -1976,7 +2105,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             };
             // skip_c: the block's row blocks hold no valid row (sparse tile); only its share of the
             // DMA issue is left
-            auto mma_block = [&](const i32x8 (&wf)[FN], const i32x8 (&xh)[HM], int fm0, auto dma_c, auto skip_c) {
+            auto mma_block = [&](const i32x8 (&wf)[FN], const i32x8 (&xh)[HM], auto fm0_c, auto dma_c, auto skip_c) {
                 constexpr bool DMA = decltype(dma_c)::value;
                 constexpr int NM = FN * HM;
                 if constexpr (decltype(skip_c)::value) {
@@ -1991,8 +2120,19 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int fn = m / HM, fm = m % HM;
-                    acc[fn][fm0 + fm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                        wf[fn], xh[fm], acc[fn][fm0 + fm], 0, 0, 0, 0, 0, 0);
+                    constexpr int FM0 = decltype(fm0_c)::value;
+                    if constexpr (MSC) {
+                        // (the byte selectors are immediates of the instruction: after unrolling fn and
+                        // fm are constants and one of the four forms is left)
+                        static_assert(FN == 2 && HM == 2, "selector forms below");
+                        if (fn == 0 && fm == 0) mfma_e4m3_scaled<0, FM0>(wf[0], xh[0], acc[0][FM0], sc_w, sc_x);
+                        else if (fn == 0) mfma_e4m3_scaled<0, FM0 + 1>(wf[0], xh[1], acc[0][FM0 + 1], sc_w, sc_x);
+                        else if (fm == 0) mfma_e4m3_scaled<1, FM0>(wf[1], xh[0], acc[1][FM0], sc_w, sc_x);
+                        else mfma_e4m3_scaled<1, FM0 + 1>(wf[1], xh[1], acc[1][FM0 + 1], sc_w, sc_x);
+                    } else {
+                        acc[fn][FM0 + fm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+                            wf[fn], xh[fm], acc[fn][FM0 + fm], 0, 0, 0, 0, 0, 0);
+                    }
                     if (DMA && (m + 1) % EVERY == 0) {
                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -2015,11 +2155,11 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 const int s2 = s1 + 1 == STAGES ? 0 : s1 + 1;
                 if (!SP) load_x1(qx1, cslot);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwa, qx0, 0, std::false_type{}, full);
+                mma_block(qwa, qx0, std::integral_constant<int, 0>{}, std::false_type{}, full);
                 __builtin_amdgcn_sched_barrier(0);
                 load_w_x0(qwb, qx0, s1);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwa, qx1, HM, std::false_type{}, sparse_c);
+                mma_block(qwa, qx1, std::integral_constant<int, HM>{}, std::false_type{}, sparse_c);
                 __builtin_amdgcn_sched_barrier(0);
                 barrier();                  // B
                 part_a = lds_base + islot * TL::STAGE_BYTES;    // pair (c+4, c+5)
@@ -2031,7 +2171,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 ikt += 2;
                 if (!SP) load_x1(qx1, s1);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwb, qx0, 0, std::integral_constant<bool, HALF == 0>{}, full);
+                mma_block(qwb, qx0, std::integral_constant<int, 0>{}, std::integral_constant<bool, HALF == 0>{}, full);
                 __builtin_amdgcn_sched_barrier(0);
                 if (!skip_wait) {
                     if (HALF == 0) wait_vmcnt<2 * L>();
@@ -2040,7 +2180,7 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 barrier();                  // A'
                 if (!LAST) load_w_x0(qwa, qx0, s2);
                 __builtin_amdgcn_sched_barrier(0);
-                mma_block(qwb, qx1, HM, std::integral_constant<bool, HALF == 1>{}, sparse_c);
+                mma_block(qwb, qx1, std::integral_constant<int, HM>{}, std::integral_constant<bool, HALF == 1>{}, sparse_c);
                 __builtin_amdgcn_sched_barrier(0);
                 cslot = s2;
             };
@@ -2098,23 +2238,45 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
             wait_vmcnt<L>();
             landed = issued - 2;
         }
+        if constexpr (MSC) mfma_results_guard();    // the last MFMAs' results are read by VALU code from here on
         FMOE_TRACE_STAMP(1);
         const TileInfo done = cur;
         cur = nxt;          // valid when another tile follows
         prefetch_next();    // nxt: the tile after that one; its row indices arrive during the epilogue
         FMOE_TRACE_STAMP(2);
 
+        // MSC: the scales of the tile that is computed next (cur, when one follows): its row indices
+        // are requested here, its scales behind the first row block of the epilogue (by then the
+        // indices have arrived: the compiler's wait for them counts that block's stores exactly),
+        // and the codes are packed at the epilogue's end, where the wait for the scale loads also
+        // covers every LDS-DMA issued before the epilogue, as the counted wait there does.
+        // (After the block's last tile cur is stale but still describes a tile of this launch:
+        // the loads stay in bounds and their result is not used.)
+        int32_t sc_idx[FM];
+        float sc_xraw[FM], sc_wraw[FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i) { sc_idx[i] = 0; sc_xraw[i] = 1.0f; }
+#pragma unroll
+        for (int i = 0; i < FN; ++i) sc_wraw[i] = 1.0f;
+        if constexpr (MSC) sc_fetch_rows(cur, sc_idx);
         auto convert_rows = [&]() __attribute__((always_inline)) {
+            if constexpr (MSC) sc_pack(sc_xraw, sc_wraw);
             rows_to_offsets(ridx_next, xoff_next);  // of the tile after the next one
         };
+        auto scales_behind_block0 = [&](int fm) __attribute__((always_inline)) {
+            if constexpr (MSC) {
+                if (fm == 0) sc_fetch_scales(cur, sc_idx, sc_xraw, sc_wraw);
+            }
+        };
+        auto hooks = make_hooks(scales_behind_block0, convert_rows);
 #ifdef FMOE_TRACE
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR, ROW_IL>(
-            p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane, convert_rows,
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, true, PAIR, XTR, ROW_IL, decltype(hooks), MSC>(
+            p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane, hooks,
             (p.trace && tile_i < 32 && (wave == 0 || wave == NW / 2)) ? tstamp + 12 : nullptr);
 #else
         static_assert(kEpilogueStoresUnconditional, "skip_wait needs an epilogue whose stores are all issued");
-        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, kEpilogueStoresUnconditional, PAIR, XTR, ROW_IL>(p, acc, done.expert, done.nt * BN_OUT, done.row0,
-                                                                done.rows_valid, wm, wn, lane, convert_rows);
+        gemm_epilogue<FM, FN, TM, TN, FP8, EPI, kEpilogueStoresUnconditional, PAIR, XTR, ROW_IL, decltype(hooks), MSC>(
+            p, acc, done.expert, done.nt * BN_OUT, done.row0, done.rows_valid, wm, wn, lane, hooks);
 #endif
 #ifdef FMOE_TRACE
         FMOE_TRACE_STAMP(3);
@@ -2181,7 +2343,7 @@ int launch_gemm(GemmParams p, hipStream_t stream) {
 int compute_units();   // CUs of the current device (gemm_api.hip)
 int lds_per_block();   // largest LDS allocation of one block on the current device (gemm_api.hip)
 
-template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false>
+template <typename TL, bool FP8, int EPI, bool WTR = false, bool KWIN = false, bool XTR = false, bool MSC = false>
 int launch_ring_cfg(GemmParams p, hipStream_t stream) {
     constexpr int bn_out = EPI == FMOE_EPI_SWIGLU ? TL::BN / 2 : TL::BN;
     p.n_tiles = (p.N + bn_out - 1) / bn_out;
@@ -2195,9 +2357,9 @@ int launch_ring_cfg(GemmParams p, hipStream_t stream) {
         // Up to 64 slices the group keeps sharing its fills and the shortened loop pays (forward
         // GEMMs of 64 experts -0.6 %, e4m3 at 128 experts -2.4 %); with 128 slices (K = 4096 in bf16,
         // 2048 rows per expert) the fills it breaks cost more than it saves (GEMM1 +1.8 %).
-        p.short_tile_rows = p.K / (FP8 ? 64 : 32) <= 64 ? TL::BM / 2 : 0;
+        p.short_tile_rows = (p.K / (FP8 ? 64 : 32) <= 64 || p.total_rows / p.E <= 2 * TL::BM) ? TL::BM / 2 : 0;
     }
-    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN, XTR>;
+    auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN, XTR, MSC>;
     static bool attr_done = false;
     if (int rc = reserve_lds(kern, TL::LDS_BYTES, attr_done)) return rc;
     // persistent: one block per CU (the LDS footprint admits no second one), a multiple of
@@ -2240,6 +2402,12 @@ int launch_ring(const GemmParams& p, hipStream_t stream) {
                 return launch_ring_cfg<TileRing5W, FP8, EPI, false, true>(p, stream);
         }
         return launch_gemm<TileBig, FP8 ? kDtE4m3 : kDtBf16, EPI, true, false>(p, stream);
+    }
+    if constexpr (FP8) {                   // power-of-two scales: applied by the MFMAs (row numbers fit 31 bits: pair_ok)
+        if (p.scale_pow2 && pair_ok && p.E <= TileRing5::kMaxExperts)
+            return launch_ring_cfg<TileRing5, FP8, EPI, false, false, false, true>(p, stream);
+        if (p.scale_pow2 && pair_ok && p.E <= TileRing5W::kMaxExperts)
+            return launch_ring_cfg<TileRing5W, FP8, EPI, false, false, false, true>(p, stream);
     }
     if (pair_ok && p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI>(p, stream);
     if (pair_ok && p.E <= TileRing5W::kMaxExperts) return launch_ring_cfg<TileRing5W, FP8, EPI>(p, stream);

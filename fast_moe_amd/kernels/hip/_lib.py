@@ -22,7 +22,7 @@ EXPORTED_SYMBOLS = (
     "fmoe_route_from_topk", "fmoe_quant_rows_e4m3", "fmoe_grouped_gemm", "fmoe_grouped_gemm_plan",
     "fmoe_combine",
     "fmoe_silu_mul", "fmoe_transpose_last2", "fmoe_jagged_transpose", "fmoe_segment_colsum",
-    "fmoe_swiglu_bwd", "fmoe_combine_bwd", "fmoe_gather_rows", "fmoe_route_topk_static",
+    "fmoe_swiglu_bwd", "fmoe_combine_bwd", "fmoe_gather_rows", "fmoe_route_topk_static", "fmoe_hbm_probe",
 )
 ROUTE_STATIC_MAX_POSITIONS, ROUTE_STATIC_MAX_EXPERTS = 1 << 20, 512
 
@@ -48,7 +48,7 @@ class GemmDesc(ctypes.Structure):
         ("aux2", c_void_p),
         ("aux_stride_row", c_int64),
         ("a_stride_k", c_int64),
-        ("a2", c_void_p), ("k2", c_int32), ("reserved1", c_int32), ("out2", c_void_p),
+        ("a2", c_void_p), ("k2", c_int32), ("scale_pow2", c_int32), ("out2", c_void_p),
     ]
 
 
@@ -110,6 +110,8 @@ def load() -> ctypes.CDLL:
     lib.fmoe_combine_bwd.argtypes = [c_void_p, c_void_p, c_int, c_int64, c_int, c_int64, c_int64, c_void_p,
                                      c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
                                      c_void_p]
+    lib.fmoe_hbm_probe.restype = c_int
+    lib.fmoe_hbm_probe.argtypes = [c_void_p, c_int64, c_int, c_int, c_void_p]
     _lib = lib
     return lib
 

@@ -211,7 +211,7 @@ class IndexSelectJaggedBmmFp8(torch.autograd.Function):
         qa, sa = ops.quant_rows_fp8(jagged)
         ctx.save_for_backward(offsets, index, jagged, weight, bias)
         return ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=index.numel(), row_index=index,
-                                index_div=index.shape[-1], bias=bias, a_scale=sa, b_scale=fp8_weight[1],
+                                index_div=index.shape[-1], bias=bias, scales_pow2=True, a_scale=sa, b_scale=fp8_weight[1],
                                 epilogue=EPI_NONE)
 
     @staticmethod
@@ -228,7 +228,7 @@ class IndexSelectJaggedBmmFp8(torch.autograd.Function):
             if weight.stride(2) != 1 and weight.stride(1) == 1:         # rows along N strided: one transposing copy
                 w_rows = ops.to_k_contiguous(weight.permute(0, 2, 1)).permute(0, 2, 1)
             qw, sw = ops.quant_rows_fp8(w_rows)                         # [E, Kin, N], [E, Kin]
-            d_rows = ops.grouped_gemm(offsets, qd, qw.permute(0, 2, 1), total_rows=R, a_scale=sd, b_scale=sw)
+            d_rows = ops.grouped_gemm(offsets, qd, qw.permute(0, 2, 1), total_rows=R, scales_pow2=True, a_scale=sd, b_scale=sw)
             d_jagged = ops.combine(d_rows, _reverse_from_index(index)).view_as(jagged)
         if need[3]:
             pad_offsets, bound = _pad_layout(offsets, R)
@@ -244,7 +244,7 @@ class IndexSelectJaggedBmmFp8(torch.autograd.Function):
             rows = torch.arange(E * M, device=dev, dtype=torch.int64) % M
             b = q_r.t().unsqueeze(0).expand(E, bound, C)                # B[e, r, c] = q_r[c, r]
             d_w = ops.grouped_gemm(seg, q_l, b, total_rows=E * M, row_index=rows, index_div=1,
-                                   a_scale=s_l, b_scale=s_r.unsqueeze(0).expand(E, C).contiguous(),
+                                   scales_pow2=True, a_scale=s_l, b_scale=s_r.unsqueeze(0).expand(E, C).contiguous(),
                                    k_window=pad_offsets, k_window_multiple=_WINDOW_MULTIPLE)
             d_w = d_w.view(E, M, C).to(weight.dtype)
             if by_n:
@@ -379,7 +379,7 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
         else:
             qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
             bmm_out = ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=jagged.shape[0], bias=bias,
-                                       a_scale=sa, b_scale=fp8_weight[1], epilogue=EPI_NONE)
+                                       scales_pow2=True, a_scale=sa, b_scale=fp8_weight[1], epilogue=EPI_NONE)
         out = ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
         ctx.save_for_backward(offsets, jagged, weight, bias, index, gating_scores, gates_index,
                               None if recompute else bmm_out, silu_rows)

@@ -283,13 +283,15 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
                  k_window_multiple: int = 0,
                  aux: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                  gate: Optional[torch.Tensor] = None,
-                 plan_only: bool = False) -> torch.Tensor:
+                 plan_only: bool = False, scales_pow2: bool = False) -> torch.Tensor:
     """Jagged GEMM, see fmoe_grouped_gemm.  ``b`` (and ``b2``) are [E, K, N] tensors of any
     strides, bf16 / fp32 / float8_e4m3fn; ``a`` is [rows, K] with contiguous rows.  Returns
     [total_rows, N] in bf16 (fp32 for fp32 operands).  ``aux`` = two tensors like the output
     that receive the SWIGLU pre-activations.  ``gate`` (bf16 [total_rows, N], with
     ``epilogue=EPI_GATED``): the result is ``silu(gate) * (A B + bias)``.  ``plan_only``: launch nothing and return the
-    _lib.PLAN_* code of the kernel this call would run (fmoe_grouped_gemm_plan)."""
+    _lib.PLAN_* code of the kernel this call would run (fmoe_grouped_gemm_plan).  ``scales_pow2``
+    (e4m3): a promise that every scale is an exact power of two, as ``quant_rows_fp8`` writes them;
+    the ring kernel then folds them into its MFMAs (fmoe_gemm_desc.scale_pow2)."""
     dev = _need_cuda("grouped_gemm", offsets, a, b, row_index, bias, b2, bias2, a_scale, b_scale, b2_scale)
     fp8 = a.dtype == FP8_DTYPE
     if not fp8 and a.dtype not in (torch.bfloat16, torch.float32):
@@ -382,6 +384,7 @@ def grouped_gemm(offsets: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, tot
     d.b_stride_e, d.b_stride_k, d.b_stride_n = b.stride()
     d.b_scale = _ptr(b_scale)
     d.b2_scale = _ptr(b2_scale)
+    d.scale_pow2 = int(bool(scales_pow2) and fp8)
     d.bias = _ptr(bias)
     d.bias2 = _ptr(bias2)
     d.bias_stride_e = bias.stride(0) if bias is not None else (bias2.stride(0) if bias2 is not None else 0)

@@ -162,7 +162,7 @@ def silu_jagged_bmm_fp8(
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=True)
     qw, sw = _weight_pair(weight.permute(0, 2, 1), fp8_weight)          # rows of [E, D_out, D_in]
     return ops.grouped_gemm(seq_offsets, qa, qw, total_rows=jagged.shape[0], bias=bias,
-                            a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
+                            scales_pow2=True, a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
 
 
 def silu_jagged_bmm_combine_fp8(
@@ -192,7 +192,7 @@ def silu_jagged_bmm_combine_fp8(
         return _ag.SiluJaggedBmmCombine.apply(offsets, jagged, weight, bias, index, reverse_index, gating_scores,
                                               gates_index, has_silu, (qw, sw), activation_checkpointing)
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
-    bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias, a_scale=sa,
+    bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias, scales_pow2=True, a_scale=sa,
                                b_scale=sw, epilogue=EPI_NONE)
     return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
 
@@ -226,5 +226,5 @@ def index_select_jagged_bmm(
         return _ag.IndexSelectJaggedBmmFp8.apply(offsets, index, jagged, weight, bias, (qw, sw))
     qa, sa = ops.quant_rows_fp8(jagged)
     return ops.grouped_gemm(offsets, qa, qw, total_rows=index.numel(), row_index=index,
-                            index_div=index.shape[-1], bias=bias, a_scale=sa, b_scale=sw,
+                            index_div=index.shape[-1], bias=bias, scales_pow2=True, a_scale=sa, b_scale=sw,
                             epilogue=EPI_NONE)

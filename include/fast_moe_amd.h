@@ -259,7 +259,14 @@ typedef struct fmoe_gemm_desc {
                                 contiguous (b_stride_n = 1), k and k2 in multiples of 128; other
                                 descriptors with a2 are turned away with FMOE_ERR_ARGUMENT */
     int32_t k2;             /* contraction length of a2 * b2                                */
-    int32_t reserved1;
+    int32_t scale_pow2;     /* FMOE_E4M3: non-zero = the caller promises that every value of a_scale,
+                                b_scale and b2_scale is an exact power of two (what
+                                fmoe_quant_rows_e4m3 writes, the convention of
+                                kernels/pytorch/quant_fp8.py:13-24).  The LDS-ring kernel then lets
+                                the MFMA instructions divide the scales out (as their E8M0 block
+                                scales) instead of its epilogue; same results.  With 0 any fp32
+                                scales are accepted.  A broken promise drops the mantissa of the
+                                scale, nothing else                                            */
     void* out2;             /* NULL, or (with a_stride_k only) a second output: offsets then
                                 describes experts of 2 * h rows each (h a multiple of 32), and
                                 rows [h, 2h) of every expert are stored to out2 + (e * h + row - h) *
@@ -317,6 +324,15 @@ int fmoe_combine(const void* value, int value_dtype, int64_t T, int K, int64_t D
  * silu_jagged_bmm_combine(has_silu=True) contracts with. */
 int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
                   fmoe_stream_t stream);
+
+/*
+ * Measurement aid with no counterpart in the reference (bench.py --hbm-ceiling): streams `bytes`
+ * of device memory at `buf` with nothing but memory accesses, so that the GB/s of the quantisers and
+ * of the merge can be read against what this part delivers to a kernel that only reads
+ * (mode 0), only writes (mode 1; the buffer is overwritten) or copies its first half to its second
+ * (mode 2).  `bytes`: a multiple of 32 KiB (64 KiB for a copy); `blocks`: grid size, 256 lanes each.
+ */
+int fmoe_hbm_probe(void* buf, int64_t bytes, int mode, int blocks, fmoe_stream_t stream);
 
 /*
  * dst[b, c, r] = src[b, r, c] for 1- or 2-byte elements: turns N-contiguous expert weights

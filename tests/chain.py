@@ -101,10 +101,10 @@ def gpu_chain(x, routing, wg, wu, wd, gates, K, fp8=False, qweights=None, want_p
         if fp8:
             (qg, sg), (qu, su), (qd, sd) = qweights
             qx, sx = ops.quant_rows_fp8(x)
-            kw1 = dict(total_rows=R, row_index=gi, index_div=K, b2=qu, epilogue=2, a_scale=sx, b_scale=sg, b2_scale=su)
+            kw1 = dict(total_rows=R, row_index=gi, index_div=K, b2=qu, epilogue=2, scales_pow2=True, a_scale=sx, b_scale=sg, b2_scale=su)
             hidden = ops.grouped_gemm(off, qx, qg, **kw1)
             qh, sh = ops.quant_rows_fp8(hidden)
-            kw2 = dict(total_rows=R, a_scale=sh, b_scale=sd)
+            kw2 = dict(total_rows=R, scales_pow2=True, a_scale=sh, b_scale=sd)
             rows = ops.grouped_gemm(off, qh, qd, **kw2)
             out.update(qx=qx, sx=sx, qh=qh, sh=sh)
             if want_plans:

@@ -887,3 +887,52 @@ def test_accumulation_error_stays_under_the_floors_the_stage_checks_use(rows):
     assert worst16 <= BF16_FLOOR / 4, f"bf16 accumulation error {worst16:.3g} of S"
     assert worst8 <= FP8_FLOOR / 4, f"e4m3 accumulation error {worst8:.3g} of S"
     assert worst8 > worst16
+
+
+@pytest.mark.parametrize("E,rows,K,N,epi,bias,gather", [
+    (8, 4096, 2048, 1408, 2, False, True),        # SwiGLU, gathered rows, last column tile partial
+    (8, 4096, 1408, 2048, 0, False, False),       # plain epilogue, rows in place
+    (8, 3000, 512, 512, 1, True, True),           # SiLU with bias
+    (128, 40000, 1024, 768, 2, True, True),       # the register-table variant for up to 256 experts
+    (6, 700, 256, 256, 0, True, False),           # short experts: tiles that run the shortened loop
+])
+def test_scales_applied_by_the_mfma_equal_scales_divided_out_in_the_epilogue(E, rows, K, N, epi, bias, gather):
+    """fmoe_gemm_desc.scale_pow2: with power-of-two scales the ring kernel lets the MFMA apply them
+    (E8M0 block scales) instead of dividing them out in its epilogue.  A power-of-two factor on
+    every product of an output element commutes with the fp32 accumulation, so the two paths must
+    agree bit for bit, also with rows and columns whose scales differ by 2^20 and with the scale of
+    an all-zero row (2^127)."""
+    from fast_moe_amd.kernels.hip import _lib, ops
+    g = torch.Generator().manual_seed(E * 7 + rows)
+    T = rows // 2 if gather else rows
+    x = torch.randn(T, K, generator=g)
+    x[::7] *= 300.0                     # other row scales
+    x[5] = 0.0                          # scale 2^127
+    x[::11] *= 2.0 ** -12
+    w = torch.randn(E, N, K, generator=g) * K ** -0.5
+    w[:, ::5] *= 64.0                   # other column scales
+    w[:, 3] = 0.0
+    w2 = torch.randn(E, N, K, generator=g) * K ** -0.5
+    qx, sx = ops.quant_rows_fp8(x.to(BF16).cuda())
+    qw, sw = ops.quant_rows_fp8(w.to(BF16).cuda())
+    qw2, sw2 = ops.quant_rows_fp8(w2.to(BF16).cuda())
+    cuts = torch.sort(torch.randint(0, rows, (E - 1,), generator=g)).values
+    if E == 6:
+        cuts = torch.tensor([100, 228, 357, 390, 650])          # 100, 128, 129, 33, 260, 50 rows
+    offsets = torch.cat([torch.zeros(1, dtype=torch.int64), cuts.to(torch.int64), torch.tensor([rows])]).cuda()
+    kw = dict(total_rows=rows, a_scale=sx, b_scale=sw, epilogue=epi)
+    if gather:
+        kw.update(row_index=torch.randint(0, T * 2, (rows,), generator=g).cuda(), index_div=2)
+    if epi == 2:
+        kw.update(b2=qw2.permute(0, 2, 1), b2_scale=sw2)
+    if bias:
+        kw.update(bias=torch.randn(E, N, generator=g).to(BF16).cuda())
+        if epi == 2:
+            kw.update(bias2=torch.randn(E, N, generator=g).to(BF16).cuda())
+    assert ops.grouped_gemm(offsets, qx, qw.permute(0, 2, 1), plan_only=True, scales_pow2=True, **kw) == _lib.PLAN_RING
+    plain = ops.grouped_gemm(offsets, qx, qw.permute(0, 2, 1), scales_pow2=False, **kw)
+    folded = ops.grouped_gemm(offsets, qx, qw.permute(0, 2, 1), scales_pow2=True, **kw)
+    again = ops.grouped_gemm(offsets, qx, qw.permute(0, 2, 1), scales_pow2=True, **kw)
+    assert torch.isfinite(plain.float()).all()
+    assert torch.equal(folded.view(torch.int16), plain.view(torch.int16))
+    assert torch.equal(again.view(torch.int16), folded.view(torch.int16))

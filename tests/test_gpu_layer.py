@@ -122,9 +122,9 @@ def test_swiglu_moe_bf16_and_fp8_composition(T, E, K, D, H):
         qd, sd = moe_fp8.quantize_expert_weights(dev(wd_v))
         qx, sx = ops.quant_rows_fp8(dev(x))
         h8 = ops.grouped_gemm(rg["offsets"], qx, qg, total_rows=T * K, row_index=rg["gate_index"], index_div=K,
-                              b2=qu, epilogue=2, a_scale=sx, b_scale=sg, b2_scale=su)
+                              b2=qu, epilogue=2, scales_pow2=True, a_scale=sx, b_scale=sg, b2_scale=su)
         qh, sh = ops.quant_rows_fp8(h8)
-        o8 = ops.grouped_gemm(rg["offsets"], qh, qd, total_rows=T * K, a_scale=sh, b_scale=sd)
+        o8 = ops.grouped_gemm(rg["offsets"], qh, qd, total_rows=T * K, scales_pow2=True, a_scale=sh, b_scale=sd)
         y8 = ops.combine(o8, rg["reverse_index"], dev(gates), rg["gate_index"])
     scale16 = ref16.float().abs().max().item()
     assert_bf16_close(y16, ref16, rtol=1e-2, atol=1e-2 * scale16, what="swiglu bf16")
@@ -235,9 +235,9 @@ def test_forward_replays_from_a_hip_graph(fp8):
         if fp8:
             qx, sx = ops.quant_rows_fp8(x)
             hid = ops.grouped_gemm(r["offsets"], qx, qg, row_index=r["gate_index"], index_div=K, b2=qu, epilogue=2,
-                                   a_scale=sx, b_scale=sg, b2_scale=su, **kw)
+                                   scales_pow2=True, a_scale=sx, b_scale=sg, b2_scale=su, **kw)
             qh, sh = ops.quant_rows_fp8(hid)
-            rows = ops.grouped_gemm(r["offsets"], qh, qd, a_scale=sh, b_scale=sd, **kw)
+            rows = ops.grouped_gemm(r["offsets"], qh, qd, scales_pow2=True, a_scale=sh, b_scale=sd, **kw)
         else:
             hid = ops.grouped_gemm(r["offsets"], x, wg, row_index=r["gate_index"], index_div=K, b2=wu, epilogue=2, **kw)
             rows = ops.grouped_gemm(r["offsets"], hid, wd, **kw)
