@@ -2357,6 +2357,8 @@ int launch_ring_cfg(GemmParams p, hipStream_t stream) {
         // Up to 64 slices the group keeps sharing its fills and the shortened loop pays (forward
         // GEMMs of 64 experts -0.6 %, e4m3 at 128 experts -2.4 %); with 128 slices (K = 4096 in bf16,
         // 2048 rows per expert) the fills it breaks cost more than it saves (GEMM1 +1.8 %).
+        // With two row tiles or fewer per expert on average there is little sharing to break, and the
+        // second tile of most experts is a short one: the shortened loop stays on whatever K is.
         p.short_tile_rows = (p.K / (FP8 ? 64 : 32) <= 64 || p.total_rows / p.E <= 2 * TL::BM) ? TL::BM / 2 : 0;
     }
     auto kern = grouped_gemm_ring_kernel<TL, FP8, EPI, WTR, KWIN, XTR, MSC>;
