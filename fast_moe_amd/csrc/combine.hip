@@ -7,6 +7,17 @@
 namespace fmoe {
 namespace {
 
+// two fp32 -> two bf16 (round to nearest even) in one v_cvt_pk_bf16_f32: the products of the merge
+// are rounded to bf16 one by one, and done with integer arithmetic that rounding is half of this
+// kernel's instructions (the kernel is then bound by its VALU work, not by the memory it reads)
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    const bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
 template <typename T>
 struct Elem;
 template <>
@@ -38,7 +49,7 @@ struct Elem<uint16_t> {
     __device__ static u32x4 pack(const float* f) {
         u32x4 r;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) r[i] = f32_to_bf16_bits(f[2 * i]) | (f32_to_bf16_bits(f[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) r[i] = cvt_pk_bf16(f[2 * i], f[2 * i + 1]);
         return r;
     }
 };
@@ -137,11 +148,20 @@ __global__ __launch_bounds__(256) void combine_kernel(const TV* __restrict__ val
                     float f[VEC];
                     if (VECTOR) Elem<TV>::unpack(raw[jj][c], f);
                     else f[0] = sv[jj][c];
+                    if constexpr (HAS_GATE && ROUND_BF16 && VEC % 2 == 0) {
 #pragma unroll
-                    for (int i = 0; i < VEC; ++i) {
-                        float p = HAS_GATE ? f[i] * wj[jj] : f[i];
-                        if (HAS_GATE && ROUND_BF16) p = round_bf16(p);
-                        acc[c][i] = acc[c][i] + p;
+                        for (int i = 0; i < VEC; i += 2) {       // products rounded to bf16 two at a time
+                            const uint32_t pk = cvt_pk_bf16(f[i] * wj[jj], f[i + 1] * wj[jj]);
+                            acc[c][i] = acc[c][i] + __uint_as_float(pk << 16);
+                            acc[c][i + 1] = acc[c][i + 1] + __uint_as_float(pk & 0xffff0000u);
+                        }
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) {
+                            float p = HAS_GATE ? f[i] * wj[jj] : f[i];
+                            if (HAS_GATE && ROUND_BF16) p = round_bf16(p);
+                            acc[c][i] = acc[c][i] + p;
+                        }
                     }
                 }
             }
