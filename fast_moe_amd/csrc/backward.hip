@@ -279,24 +279,22 @@ __global__ __launch_bounds__(256) void swiglu_bwd_bf16x8_kernel(const uint16_t* 
     u32x4 vu = {0, 0, 0, 0}, og, ou = {0, 0, 0, 0};
     if (GATED) vu = reinterpret_cast<const u32x4*>(u)[i];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        uint32_t rg = 0, ru = 0;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const float gv = bf16_bits_to_f32((vg[q] >> (16 * h)) & 0xffffu);
-            const float d = bf16_bits_to_f32((vd[q] >> (16 * h)) & 0xffffu);
-            const float s = sigmoid_f32(gv);
-            const float dsilu = s * (1.0f + gv * (1.0f - s));
-            if (GATED) {
-                const float uv = bf16_bits_to_f32((vu[q] >> (16 * h)) & 0xffffu);
-                ru |= f32_to_bf16_bits(d * round_bf16(gv * s)) << (16 * h);
-                rg |= f32_to_bf16_bits(round_bf16(d * uv) * dsilu) << (16 * h);
-            } else {
-                rg |= f32_to_bf16_bits(d * dsilu) << (16 * h);
-            }
+    for (int q = 0; q < 4; ++q) {       // two elements at a time: every bf16 rounding is one pack instruction
+        const float g0 = bf16_bits_to_f32(vg[q] & 0xffffu), g1 = __uint_as_float(vg[q] & 0xffff0000u);
+        const float d0 = bf16_bits_to_f32(vd[q] & 0xffffu), d1 = __uint_as_float(vd[q] & 0xffff0000u);
+        const float s0 = sigmoid_f32(g0), s1 = sigmoid_f32(g1);
+        const float ds0 = s0 * (1.0f + g0 * (1.0f - s0)), ds1 = s1 * (1.0f + g1 * (1.0f - s1));
+        if (GATED) {
+            const float u0 = bf16_bits_to_f32(vu[q] & 0xffffu), u1 = __uint_as_float(vu[q] & 0xffff0000u);
+            float a0 = g0 * s0, a1 = g1 * s1;       // silu(g), rounded as the forward rounds it
+            round_bf16_pair(a0, a1);
+            ou[q] = cvt_pk_bf16(d0 * a0, d1 * a1);
+            float b0 = d0 * u0, b1 = d1 * u1;
+            round_bf16_pair(b0, b1);
+            og[q] = cvt_pk_bf16(b0 * ds0, b1 * ds1);
+        } else {
+            og[q] = cvt_pk_bf16(d0 * ds0, d1 * ds1);
         }
-        og[q] = rg;
-        ou[q] = ru;
     }
     reinterpret_cast<u32x4*>(dg)[o] = og;
     if (GATED) reinterpret_cast<u32x4*>(du)[o] = ou;
@@ -361,10 +359,12 @@ __global__ __launch_bounds__(256) void combine_bwd_kernel(const T* __restrict__ 
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float d0 = bf16_bits_to_f32(vd[q] & 0xffffu), d1 = __uint_as_float(vd[q] & 0xffff0000u);
-                o[q] = f32_to_bf16_bits(d0 * w) | (f32_to_bf16_bits(d1 * w) << 16);
+                o[q] = cvt_pk_bf16(d0 * w, d1 * w);
                 if (d_gates) {
-                    dot += round_bf16(bf16_bits_to_f32(vv[q] & 0xffffu) * d0);
-                    dot += round_bf16(__uint_as_float(vv[q] & 0xffff0000u) * d1);
+                    float p0 = bf16_bits_to_f32(vv[q] & 0xffffu) * d0, p1 = __uint_as_float(vv[q] & 0xffff0000u) * d1;
+                    round_bf16_pair(p0, p1);
+                    dot += p0;
+                    dot += p1;
                 }
             }
             __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(dvr + c));

@@ -7,17 +7,6 @@
 namespace fmoe {
 namespace {
 
-// two fp32 -> two bf16 (round to nearest even) in one v_cvt_pk_bf16_f32: the products of the merge
-// are rounded to bf16 one by one, and done with integer arithmetic that rounding is half of this
-// kernel's instructions (the kernel is then bound by its VALU work, not by the memory it reads)
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
-    const f32x2_t v = {lo, hi};
-    const bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
-    return __builtin_bit_cast(uint32_t, r);
-}
-
 template <typename T>
 struct Elem;
 template <>

@@ -47,6 +47,24 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// two fp32 -> two bf16 (round to nearest even) in one v_cvt_pk_bf16_f32, `lo` in the low half: for
+// loops that round every element they touch (with the integer sequence above, which also keeps a
+// NaN's payload, the rounding is most of such a loop's instructions and the loop is bound by them,
+// not by the memory it streams)
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ uint32_t cvt_pk_bf16(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    const bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+}
+// both values rounded to bf16 and back
+__device__ __forceinline__ void round_bf16_pair(float& a, float& b) {
+    const uint32_t pk = cvt_pk_bf16(a, b);
+    a = __uint_as_float(pk << 16);
+    b = __uint_as_float(pk & 0xffff0000u);
+}
+
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
 // round(silu(x)) to bf16 for a bf16-valued x, equal on every one of the 65536 inputs to what
