@@ -548,8 +548,8 @@ def sustained(fn, seconds, sampler_period=0.25):
 
 def hbm_ceiling(gib=4, reps=20):
     """GB/s of kernels that do nothing but memory accesses over `gib` GiB (far beyond the 256 MB
-    last-level cache): the library's probe kernel (16-byte accesses, eight in flight per lane, at
-    two grid sizes) and torch's own reduction, fill and copy.  The fraction-of-HBM figures of the
+    last-level cache): the library's probe kernel (16-byte accesses, one, two or eight per lane)
+    and torch's own reduction, fill and copy.  The fraction-of-HBM figures of the
     quantisers and of the merge are to be read against these, not only against the 8 TB/s of the
     data sheet."""
     from fast_moe_amd.kernels.hip import _lib
@@ -561,17 +561,17 @@ def hbm_ceiling(gib=4, reps=20):
     stream = torch.cuda.current_stream(dev)
     out = {"bytes": nbytes, "launches": reps}
 
-    def probe(mode, blocks):
-        _lib.check(lib.fmoe_hbm_probe(buf.data_ptr(), nbytes, mode, blocks, stream.cuda_stream), "fmoe_hbm_probe")
+    def probe(mode, per_lane):
+        _lib.check(lib.fmoe_hbm_probe(buf.data_ptr(), nbytes, mode, per_lane, stream.cuda_stream), "fmoe_hbm_probe")
 
-    for name, mode, moved in (("read", 0, nbytes), ("write", 1, nbytes), ("copy", 2, nbytes)):
-        for blocks in (2048, 32768):
-            fn = lambda: probe(mode, blocks)
+    for name, mode in (("read", 0), ("write", 1), ("copy", 2)):
+        for per_lane in (1, 2, 8):
+            fn = lambda: probe(mode, per_lane)
             fn()
             torch.cuda.synchronize()
             ms = time_region(fn, reps, stream)
-            out[f"probe_{name}_{blocks}_blocks"] = {"ms": round(ms, 4), "gbs": round(moved / ms / 1e6, 1),
-                                                    "frac_hbm": round(moved / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            out[f"probe_{name}_{per_lane}_per_lane"] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                                                        "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
     as_f32, half = buf.view(torch.float32), nbytes // 2
     for name, fn, moved in (("torch_sum_fp32", lambda: as_f32.sum(), nbytes),
                             ("torch_fill", lambda: buf.fill_(1), nbytes),

@@ -84,36 +84,37 @@ __global__ __launch_bounds__(256) void transpose_kernel(const T* __restrict__ sr
 }
 
 // HBM probe: what this part reads and writes per second when nothing else limits a kernel.
-// Blocks of 256 lanes take 32 KB pieces of the buffer round robin; a lane has eight 16-byte
-// accesses in flight.  READ: non-temporal loads folded into a value that is stored only if it
-// takes a value no buffer produces in practice (the loads cannot be dropped).  WRITE: 16-byte
-// stores of a pattern.  COPY: first half of the buffer to the second.
-template <int MODE>
-__global__ __launch_bounds__(256) void hbm_probe_kernel(u32x4* __restrict__ buf, int64_t pieces, uint32_t* sink) {
-    constexpr int PER = 8;                      // 16-byte accesses per lane and piece: 256 * 8 * 16 B = 32 KB
-    u32x4 acc = {0, 0, 0, 0};
-    const int64_t half = pieces * 256 * PER;    // COPY: the second half starts here (in 16-byte units)
-    for (int64_t pc = blockIdx.x; pc < pieces; pc += gridDim.x) {
-        u32x4* base = buf + pc * 256 * PER + threadIdx.x;
-        if (MODE == 0) {
-            u32x4 v[PER];
+// One-shot grid: block b owns piece b of 256 * PER * 16 bytes, lane l the 16-byte words
+// l, l + 256, ... of it (every access instruction of a wave covers 1 KB of contiguous memory).
+// READ: non-temporal loads folded into a value that is stored only if it takes a value no
+// buffer produces in practice (the loads cannot be dropped).  WRITE: 16-byte stores of a
+// pattern.  COPY: first half of the buffer to the second.  PER = accesses per lane: reads want
+// several in flight, writes are fastest with one store per lane and many short waves.
+template <int MODE, int PER>
+__global__ __launch_bounds__(256) void hbm_probe_kernel(u32x4* __restrict__ buf, int64_t n16, int64_t half16,
+                                                        uint32_t* sink) {
+    const int64_t i0 = (int64_t)blockIdx.x * 256 * PER + threadIdx.x;
+    u32x4 v[PER];
+    if (MODE != 1) {
 #pragma unroll
-            for (int i = 0; i < PER; ++i) v[i] = __builtin_nontemporal_load(base + i * 256);
-#pragma unroll
-            for (int i = 0; i < PER; ++i) acc ^= v[i];
-        } else if (MODE == 1) {
-            const uint32_t x = (uint32_t)pc;
-#pragma unroll
-            for (int i = 0; i < PER; ++i) base[i * 256] = u32x4{x, x + 1, x + 2, x + 3};
-        } else {
-            u32x4 v[PER];
-#pragma unroll
-            for (int i = 0; i < PER; ++i) v[i] = __builtin_nontemporal_load(base + i * 256);
-#pragma unroll
-            for (int i = 0; i < PER; ++i) base[half + i * 256] = v[i];
+        for (int i = 0; i < PER; ++i) {
+            const int64_t idx = i0 + (int64_t)i * 256;
+            v[i] = idx < n16 ? __builtin_nontemporal_load(buf + idx) : u32x4{0, 0, 0, 0};
         }
     }
-    if (MODE == 0 && (acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) *sink = acc[0];
+    if (MODE == 0) {
+        u32x4 acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < PER; ++i) acc ^= v[i];
+        if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) *sink = acc[0];
+    } else {
+        const uint32_t x = (uint32_t)blockIdx.x * 2654435761u + threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int64_t idx = i0 + (int64_t)i * 256;
+            if (idx < n16) buf[(MODE == 2 ? half16 : 0) + idx] = MODE == 2 ? v[i] : u32x4{x, x ^ 0x5bd1e995u, x + i, ~x};
+        }
+    }
 }
 
 }  // namespace
@@ -121,21 +122,23 @@ __global__ __launch_bounds__(256) void hbm_probe_kernel(u32x4* __restrict__ buf,
 
 using namespace fmoe;
 
-extern "C" int fmoe_hbm_probe(void* buf, int64_t bytes, int mode, int blocks, fmoe_stream_t stream) {
+extern "C" int fmoe_hbm_probe(void* buf, int64_t bytes, int mode, int per_lane, fmoe_stream_t stream) {
     FMOE_REQUIRE(buf && aligned16(buf), "fmoe_hbm_probe: buf must be a 16-byte aligned device pointer");
     FMOE_REQUIRE(mode >= 0 && mode <= 2, "fmoe_hbm_probe: mode must be 0 (read), 1 (write) or 2 (copy)");
-    const int64_t piece = 256 * 8 * 16;
-    const int64_t span = mode == 2 ? bytes / 2 : bytes;
-    FMOE_REQUIRE(bytes >= 2 * piece && span % piece == 0,
-                 "fmoe_hbm_probe: bytes must be a multiple of %lld (twice that for a copy)", (long long)piece);
-    FMOE_REQUIRE(blocks >= 1 && blocks <= (1 << 20), "fmoe_hbm_probe: 1 .. 2^20 blocks");
-    const int64_t pieces = span / piece;
+    FMOE_REQUIRE(per_lane == 1 || per_lane == 2 || per_lane == 4 || per_lane == 8,
+                 "fmoe_hbm_probe: 1, 2, 4 or 8 accesses per lane");
+    FMOE_REQUIRE(bytes >= 32 && bytes % 32 == 0, "fmoe_hbm_probe: bytes must be a multiple of 32");
+    const int64_t n16 = (mode == 2 ? bytes / 2 : bytes) / 16;
+    const int64_t grid = (n16 + 256 * (int64_t)per_lane - 1) / (256 * (int64_t)per_lane);
+    FMOE_REQUIRE(grid < ((int64_t)1 << 31), "fmoe_hbm_probe: buffer too large");
     u32x4* b = (u32x4*)buf;
-    uint32_t* sink = (uint32_t*)buf;
     hipStream_t s = (hipStream_t)stream;
-    if (mode == 0) hbm_probe_kernel<0><<<blocks, 256, 0, s>>>(b, pieces, sink);
-    else if (mode == 1) hbm_probe_kernel<1><<<blocks, 256, 0, s>>>(b, pieces, sink);
-    else hbm_probe_kernel<2><<<blocks, 256, 0, s>>>(b, pieces, sink);
+#define FMOE_PROBE(M, P)                                                                      \
+    if (mode == M && per_lane == P) hbm_probe_kernel<M, P><<<(unsigned)grid, 256, 0, s>>>(b, n16, n16, (uint32_t*)buf)
+    FMOE_PROBE(0, 1); FMOE_PROBE(0, 2); FMOE_PROBE(0, 4); FMOE_PROBE(0, 8);
+    FMOE_PROBE(1, 1); FMOE_PROBE(1, 2); FMOE_PROBE(1, 4); FMOE_PROBE(1, 8);
+    FMOE_PROBE(2, 1); FMOE_PROBE(2, 2); FMOE_PROBE(2, 4); FMOE_PROBE(2, 8);
+#undef FMOE_PROBE
     return check_launch("fmoe_hbm_probe");
 }
 

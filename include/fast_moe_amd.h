@@ -330,9 +330,10 @@ int fmoe_silu_mul(const void* a, const void* b, void* out, int dtype, int64_t n,
  * of device memory at `buf` with nothing but memory accesses, so that the GB/s of the quantisers and
  * of the merge can be read against what this part delivers to a kernel that only reads
  * (mode 0), only writes (mode 1; the buffer is overwritten) or copies its first half to its second
- * (mode 2).  `bytes`: a multiple of 32 KiB (64 KiB for a copy); `blocks`: grid size, 256 lanes each.
+ * (mode 2).  `per_lane` (1, 2, 4 or 8): 16-byte accesses per lane; the grid follows from it
+ * (256 lanes per block).  `bytes`: a multiple of 32.
  */
-int fmoe_hbm_probe(void* buf, int64_t bytes, int mode, int blocks, fmoe_stream_t stream);
+int fmoe_hbm_probe(void* buf, int64_t bytes, int mode, int per_lane, fmoe_stream_t stream);
 
 /*
  * dst[b, c, r] = src[b, r, c] for 1- or 2-byte elements: turns N-contiguous expert weights
