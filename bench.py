@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_bf16|c4_fp8|c2_bf16|c5_bf16|c5_fp8]
                     [--tokens T] [--no-cpu-baseline] [--no-extra] [--sample-clock] [--dense-reference]
-                    [--hbm-ceiling]
+                    [--hbm-ceiling] [--tile-trace]
 
 A step is one forward pass of the hot path over one batch of synthetic input that is
 already resident in HBM: top-k routing from the gate probabilities, the gather +
@@ -643,6 +643,57 @@ def sustained_section(w, sample_clock, dense_reference, seconds=3.0):
     return out
 
 
+def tile_trace(w):
+    """Where a tile's time goes inside the ring kernel, from a library built with -DFMOE_TRACE
+    (`python -m fast_moe_amd.build --out fast_moe_amd/libfastmoe_hip_trace.so -DFMOE_TRACE`, run with
+    FMOE_LIB_PATH=fast_moe_amd/libfastmoe_hip_trace.so): waves 0 and 4 of every block stamp the
+    100 MHz real-time counter at a tile's start, the end of its main loop, after the next tile has
+    been located and at the end of the epilogue (plus the row blocks inside the epilogue); the
+    stamps of one launch of each GEMM are averaged over the tiles that have a predecessor and a
+    successor in their block.  Stamped builds run slower than the product: the split is the result."""
+    import numpy as np
+    dev = torch.device("cuda:0")
+    inp = make_inputs(w, dev)
+    path = GpuPath(w, inp)
+    path.step()
+    path.step()
+    torch.cuda.synchronize()
+    grid = torch.cuda.get_device_properties(0).multi_processor_count // 8 * 8
+    out = {}
+    for which in ("gemm1", "gemm2"):
+        buf = torch.zeros(3 * grid * 32 * 2 * 8, dtype=torch.int64, device=dev)
+        fn = getattr(path, which)
+        fn()
+        torch.cuda.synchronize()
+        os.environ["FMOE_TRACE_PTR"] = hex(buf.data_ptr())
+        try:
+            fn()
+            torch.cuda.synchronize()
+        finally:
+            del os.environ["FMOE_TRACE_PTR"]
+        full = buf.cpu().numpy().reshape(3, grid, 32, 2, 8).astype(np.float64)
+        t, inner = full[0], full[2]
+        ntiles = (t[:, :, 0, 0] > 0).sum(1)
+        if ntiles.max() == 0:
+            return {"unavailable": "no stamps: the loaded library was not built with -DFMOE_TRACE"}
+        groups = {}
+        for g in (0, 1):
+            rows = []
+            for b in range(grid):
+                for i in range(1, int(ntiles[b]) - 1):
+                    r, q = t[b, i, g], inner[b, i, g]
+                    rows.append([r[1] - r[0], r[2] - r[1], r[3] - r[2], t[b, i + 1, g, 0] - r[3],
+                                 q[0] - r[2], q[4] - q[0], r[3] - q[4]])
+            m = np.mean(np.array(rows), axis=0) / 100.0       # 100 MHz ticks -> microseconds
+            groups[f"waves_{'0_3' if g == 0 else '4_7'}"] = {
+                "main_loop_us": round(m[0], 2), "locate_next_and_prefetch_us": round(m[1], 2),
+                "epilogue_us": round(m[2], 2), "epilogue_end_to_next_tile_start_us": round(m[3], 2),
+                "epilogue_before_first_row_block_us": round(m[4], 2), "epilogue_row_blocks_us": round(m[5], 2),
+                "epilogue_after_last_row_block_us": round(m[6], 2), "tiles_averaged": len(rows)}
+        out[which] = dict(groups, k_slices=int(t[0, 0, 0, 6]), tiles_per_block_max=int(ntiles.max()))
+    return out
+
+
 def with_wq(entry, timing, flops):
     """fp8 workloads: the step of the default operator path (weight quantisation inside) beside the
     headline step (weights quantised once)."""
@@ -676,6 +727,9 @@ def main():
     ap.add_argument("--hbm-ceiling", action="store_true",
                     help="also stream 4 GiB with kernels that only read, only write, and copy (fmoe_hbm_probe, and "
                          "torch's sum / fill_ / copy_ beside them): what the part gives a memory-bound kernel")
+    ap.add_argument("--tile-trace", action="store_true",
+                    help="per-tile split of the ring GEMMs (main loop / locate / epilogue) from a -DFMOE_TRACE build of "
+                         "the library loaded through FMOE_LIB_PATH; see tile_trace()")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 512 MiB device copy, for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
@@ -757,6 +811,8 @@ def main():
         line["sustained"] = sustained_section(w, args.sample_clock, args.dense_reference)
     if args.hbm_ceiling:
         line["hbm_ceiling"] = hbm_ceiling()
+    if args.tile_trace:
+        line["tile_trace"] = tile_trace(w)
     if args.calibrate_copy:      # a kernel of known traffic: 512 MiB read + 512 MiB written
         src = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)

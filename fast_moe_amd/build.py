@@ -1,6 +1,10 @@
 """Builds libfastmoe_hip.so (gfx950) from fast_moe_amd/csrc with hipcc, in-tree.
 
     python -m fast_moe_amd.build            # compile every translation unit and link
+    python -m fast_moe_amd.build --out fast_moe_amd/libfastmoe_hip_trace.so -DFMOE_TRACE
+                                            # a second library beside it (here: the debug build whose
+                                            # ring kernel records per-tile time stamps; load it with
+                                            # FMOE_LIB_PATH=<that file>, see bench.py --tile-trace)
 """
 from __future__ import annotations
 
@@ -32,8 +36,8 @@ def _hipcc() -> str:
     return "hipcc"
 
 
-def _compile(src: str, extra) -> str:
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+def _compile(src: str, extra, obj_dir: str = OBJ_DIR) -> str:
+    obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
     cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -41,18 +45,26 @@ def _compile(src: str, extra) -> str:
     return obj
 
 
-def build(extra_flags=(), jobs: int = 8, verbose: bool = True) -> str:
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def build(extra_flags=(), jobs: int = 8, verbose: bool = True, out: str = LIB_PATH) -> str:
+    # (a library under another name keeps its objects apart from the product's)
+    obj_dir = OBJ_DIR if os.path.abspath(out) == LIB_PATH else os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(out))[0])
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(SOURCES)))) as pool:
-        objs = list(pool.map(lambda s: _compile(s, list(extra_flags)), SOURCES))
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs]
+        objs = list(pool.map(lambda s: _compile(s, list(extra_flags), obj_dir), SOURCES))
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stdout}\n{res.stderr}")
     if verbose:
-        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH) / 1e6:.1f} MB)")
-    return LIB_PATH
+        print(f"built {out} ({os.path.getsize(out) / 1e6:.1f} MB)")
+    return out
 
 
 if __name__ == "__main__":
-    build(extra_flags=sys.argv[1:])
+    args = sys.argv[1:]
+    target = LIB_PATH
+    if "--out" in args:
+        i = args.index("--out")
+        target = os.path.abspath(args[i + 1])
+        del args[i:i + 2]
+    build(extra_flags=args, out=target)

@@ -10,7 +10,8 @@ import os
 from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint8, c_void_p
 
 _PKG_DIR = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-LIB_PATH = os.path.join(_PKG_DIR, "libfastmoe_hip.so")
+# (FMOE_LIB_PATH: another build of the same library, e.g. the -DFMOE_TRACE debug build)
+LIB_PATH = os.environ.get("FMOE_LIB_PATH") or os.path.join(_PKG_DIR, "libfastmoe_hip.so")
 
 FMOE_F32, FMOE_BF16, FMOE_E4M3 = 0, 1, 2
 EPI_NONE, EPI_SILU, EPI_SWIGLU, EPI_GATED = 0, 1, 2, 3
