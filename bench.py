@@ -54,7 +54,7 @@ def measured_traffic_bytes(workload):
     text = open(path).read()
     vals = {}
     for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        m = re.search(r"^\s*gemm_ring\S* fp8=\w+ epi=2\s+" + counter + r"=([0-9.e+]+)\s*$", text, re.M)
+        m = re.search(r"^\s*gemm_ring\S* fp8=\w+ epi=2(?: msc)?\s+" + counter + r"=([0-9.e+]+)\s*$", text, re.M)
         if not m:
             return None
         vals[counter] = float(m.group(1))

@@ -1,6 +1,7 @@
-// OCP e4m3 instantiations of the jagged GEMM (v_mfma_f32_32x32x64_f8f6f4, both
-// operand formats = e4m3, unit block scales; the row-wise power-of-two scales
-// are divided out in the epilogue).
+// OCP e4m3 instantiations of the jagged GEMM (v_mfma_scale_f32_32x32x64_f8f6f4, both
+// operand formats = e4m3).  Row-wise scales the caller declares to be exact powers of
+// two (fmoe_gemm_desc.scale_pow2) are applied by the MFMAs as E8M0 block scales on the
+// ring and streaming kernels; any other scales are divided out in the epilogue.
 #include "gemm_kernel.h"
 
 namespace fmoe {

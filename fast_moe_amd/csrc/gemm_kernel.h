@@ -2,7 +2,7 @@
 // bf16 or OCP-e4m3 operands, fp32 MFMA accumulation, fused bias / SiLU / SwiGLU
 // epilogue.  Shared by gemm_bf16.hip and gemm_fp8.hip.
 //
-// Two kernels share the tile geometry, the scheduler and the epilogue:
+// Three kernels share the scheduler and the epilogue:
 //
 //   grouped_gemm_ring_kernel   the fast path.  Persistent (one block per CU), 256 x 256 tiles,
 //       8 wavefronts.  Operand K-slices of 64 bytes per row travel global -> LDS with
@@ -12,9 +12,18 @@
 //       LDS (5 slots), slices are fetched in pairs as full 128-byte lines and the K loop is
 //       a software pipeline of 8-MFMA blocks (see RingCfg); otherwise 4 slots, one slice at
 //       a time, schedule tables in LDS.
+//   grouped_gemm_stream_kernel experts with a handful of rows (the weights are streamed once
+//       and that stream is the cost).  Persistent 64 x 256 tiles, 4 wavefronts, two blocks per
+//       CU; a K-slice travels global -> registers -> LDS while the previous one is multiplied,
+//       and the next tile's first slice is loaded before the current tile's epilogue, so the
+//       weight stream does not stop at tile boundaries.
 //   grouped_gemm_kernel        register-staged, double-buffered LDS; serves everything the
-//       ring kernel does not: arbitrary B strides and K / N tails (element loads), SiLU
-//       applied to A on load, and short 64-row tiles for experts with a handful of rows.
+//       other two do not: arbitrary B strides and K / N tails (element loads), SiLU applied
+//       to A on load, fp32 operands.
+//
+// e4m3 row-wise scales that are exact powers of two (GemmParams::scale_pow2) are handed to
+// v_mfma_scale_f32_32x32x64_f8f6f4 as E8M0 codes of their reciprocals instead of being divided
+// out in the epilogue (ring and streaming kernels; template parameter MSC).
 //
 // Mapping to the hardware
 //   * LDS rows are XOR-swizzled in 16-byte chunks so that the ds_read_b128 of an MFMA
