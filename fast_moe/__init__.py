@@ -4,7 +4,8 @@
 second copy), so that code written against meta-recsys/fast_moe's operator path imports
 unchanged.  ``fast_moe.dev_settings`` is there as well, and ``fast_moe.kernels.triton.triton_moe``
 names the two option dataclasses the reference's callers import from it (the HIP operators accept
-and ignore them).  Nothing else of the reference's package is provided here.
+and ignore them), ``fast_moe.utils.enums`` the three option enumerations.  Nothing else of the
+reference's package is provided here.
 """
 import importlib
 import sys
@@ -30,4 +31,11 @@ _triton.triton_moe = _triton_moe
 sys.modules[_triton.__name__] = _triton
 sys.modules[_triton_moe.__name__] = _triton_moe
 
-__all__ = ["FastMoELayer", "GatingNetwork", "KernelType", "__version__"]
+# the option enumerations under the module path the reference keeps them at (utils/enums.py)
+_enums = types.ModuleType(__name__ + ".utils.enums")
+_enums.__doc__ = "ExpertType, RouterChoice, LossType (defined in fast_moe_amd.utils)."
+from fast_moe_amd.utils import ExpertType, LossType, RouterChoice  # noqa: E402
+_enums.ExpertType, _enums.RouterChoice, _enums.LossType = ExpertType, RouterChoice, LossType
+sys.modules[_enums.__name__] = _enums
+
+__all__ = ["FastMoELayer", "GatingNetwork", "KernelType", "ExpertType", "RouterChoice", "LossType", "__version__"]

@@ -298,6 +298,13 @@ def test_imports_of_the_reference_test_files_resolve():
     set_verbose_level(0)
     assert callable(fx_infer_max_len) and callable(fx_torch_zeros_like) and callable(to_fp32_if_pytorch_kernel)
     assert FastMoELayer and MRNOutput and SGConfig and KernelType.HIP
+    # kernels/tests/mrn_test.py:24 (utils/enums.py:10-26: member names and values)
+    from fast_moe.utils.enums import ExpertType, LossType, RouterChoice
+    from fast_moe import ExpertType as root_expert_type
+    assert root_expert_type is ExpertType
+    assert [(m.name, m.value) for m in ExpertType] == [("MLP", "MLP"), ("FFN", "FFN"), ("FFNBIAS", "FFN_WITH_BIAS")]
+    assert [(m.name, m.value) for m in RouterChoice] == [("TopK", "TOP_K"), ("Vanilla", "VANILLA")]
+    assert [(m.name, m.value) for m in LossType] == [("LB", "LOAD_BALANCE"), ("MI", "MUTAL_INFORMATION")]
 
 
 def test_combine_helper_opens_the_reference_profiler_range():
