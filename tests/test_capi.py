@@ -247,7 +247,7 @@ def test_reference_helper_names_import_without_a_gpu():
     utils/configs.py:13-36)."""
     import torch
     from fast_moe_amd.kernels.utils import KernelType, fx_infer_max_len, fx_torch_zeros_like, to_fp32_if_pytorch_kernel
-    from fast_moe_amd.utils.configs import MRNOutput, SGConfig
+    from fast_moe.utils.configs import MRNOutput, SGConfig
     assert fx_infer_max_len(torch.tensor([3, 9, 2])) == 9
     assert fx_torch_zeros_like(torch.ones(2, 3), torch.bfloat16).dtype == torch.bfloat16
     assert to_fp32_if_pytorch_kernel(torch.ones(1, dtype=torch.bfloat16), KernelType.HIP).dtype == torch.bfloat16
