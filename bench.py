@@ -672,7 +672,7 @@ def tile_trace(w):
         finally:
             del os.environ["FMOE_TRACE_PTR"]
         full = buf.cpu().numpy().reshape(3, grid, 32, 2, 8).astype(np.float64)
-        t, inner = full[0], full[2]
+        t, steps, inner = full[0], full[1], full[2]
         ntiles = (t[:, :, 0, 0] > 0).sum(1)
         if ntiles.max() == 0:
             return {"unavailable": "no stamps: the loaded library was not built with -DFMOE_TRACE"}
@@ -682,14 +682,25 @@ def tile_trace(w):
             for b in range(grid):
                 for i in range(1, int(ntiles[b]) - 1):
                     r, q = t[b, i, g], inner[b, i, g]
+                    d = steps[b, i, g]      # after double steps 0..3, before the second last, before the last
+                    mid = r[6] / 2 - 6      # double steps between the fourth and the second last
                     rows.append([r[1] - r[0], r[2] - r[1], r[3] - r[2], t[b, i + 1, g, 0] - r[3],
-                                 q[0] - r[2], q[4] - q[0], r[3] - q[4]])
+                                 q[0] - r[2], q[4] - q[0], r[3] - q[4],
+                                 d[0] - r[0], d[1] - d[0], d[2] - d[1], d[3] - d[2],
+                                 (d[4] - d[3]) / mid if mid > 0 else 0.0, d[5] - d[4], r[1] - d[5]])
             m = np.mean(np.array(rows), axis=0) / 100.0       # 100 MHz ticks -> microseconds
             groups[f"waves_{'0_3' if g == 0 else '4_7'}"] = {
                 "main_loop_us": round(m[0], 2), "locate_next_and_prefetch_us": round(m[1], 2),
                 "epilogue_us": round(m[2], 2), "epilogue_end_to_next_tile_start_us": round(m[3], 2),
                 "epilogue_before_first_row_block_us": round(m[4], 2), "epilogue_row_blocks_us": round(m[5], 2),
-                "epilogue_after_last_row_block_us": round(m[6], 2), "tiles_averaged": len(rows)}
+                "epilogue_after_last_row_block_us": round(m[6], 2),
+                # the main loop by double step (a pair of K-slices): the first four, the average of
+                # those in the middle, the last two (the last one ends with the wait for the tile's
+                # own LDS-DMA stream)
+                "double_steps_first_four_us": [round(v, 2) for v in m[7:11]],
+                "double_step_middle_us": round(m[11], 3),
+                "double_steps_last_two_us": [round(v, 2) for v in m[12:14]],
+                "tiles_averaged": len(rows)}
         out[which] = dict(groups, k_slices=int(t[0, 0, 0, 6]), tiles_per_block_max=int(ntiles.max()))
     return out
 
