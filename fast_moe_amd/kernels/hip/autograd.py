@@ -211,8 +211,8 @@ class IndexSelectJaggedBmmFp8(torch.autograd.Function):
         qa, sa = ops.quant_rows_fp8(jagged)
         ctx.save_for_backward(offsets, index, jagged, weight, bias)
         return ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=index.numel(), row_index=index,
-                                index_div=index.shape[-1], bias=bias, scales_pow2=True, a_scale=sa, b_scale=fp8_weight[1],
-                                epilogue=EPI_NONE)
+                                index_div=index.shape[-1], bias=bias, scales_pow2=ops.scales_are_pow2(sa, fp8_weight[1]),
+                                a_scale=sa, b_scale=fp8_weight[1], epilogue=EPI_NONE)
 
     @staticmethod
     def backward(ctx, dout):
@@ -379,7 +379,8 @@ class SiluJaggedBmmCombine(torch.autograd.Function):
         else:
             qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
             bmm_out = ops.grouped_gemm(offsets, qa, fp8_weight[0], total_rows=jagged.shape[0], bias=bias,
-                                       scales_pow2=True, a_scale=sa, b_scale=fp8_weight[1], epilogue=EPI_NONE)
+                                       scales_pow2=ops.scales_are_pow2(sa, fp8_weight[1]), a_scale=sa,
+                                       b_scale=fp8_weight[1], epilogue=EPI_NONE)
         out = ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
         ctx.save_for_backward(offsets, jagged, weight, bias, index, gating_scores, gates_index,
                               None if recompute else bmm_out, silu_rows)

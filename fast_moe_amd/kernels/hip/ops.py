@@ -192,7 +192,18 @@ def quant_rows_fp8(a: torch.Tensor, apply_silu: bool = False, reciprocal_scale: 
         q = q[0]
     elif a.ndim > 3:
         q = q.view(shape)
-    return q, scale.view(shape[:-1])
+    scale = scale.view(shape[:-1])
+    scale._fmoe_pow2 = scale._version       # (see scales_are_pow2)
+    return q, scale
+
+
+def scales_are_pow2(*scales: torch.Tensor) -> bool:
+    """True when every scale tensor is one this module's quantiser returned (that very tensor object):
+    those hold exact powers of two (kernels/pytorch/quant_fp8.py:13-24), which is what
+    ``grouped_gemm(scales_pow2=True)`` relies on.  A tensor of any other origin (a caller's own
+    quantisation handed in as ``fp8_weight``, a slice, a copy) is not vouched for, and the GEMM then
+    divides the scales out in its epilogue, which is right for any positive scale."""
+    return all(getattr(s, "_fmoe_pow2", None) == s._version for s in scales)      # (and not written to since)
 
 
 def to_k_contiguous(w: torch.Tensor) -> torch.Tensor:

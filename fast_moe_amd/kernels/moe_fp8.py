@@ -108,7 +108,9 @@ def cached_quantize_expert_weights(weight: torch.Tensor) -> Tuple[torch.Tensor, 
 
 def _weight_pair(weight: torch.Tensor, fp8_weight) -> Tuple[torch.Tensor, torch.Tensor]:
     """The (e4m3 [E, K, N], scale [E, N]) pair of ``weight``: the caller's, checked for shape, or a
-    fresh quantisation."""
+    fresh quantisation.  (A caller's own pair may carry any positive scales: the GEMM takes the
+    scales for powers of two only when they are tensors this package's quantiser returned,
+    ``ops.scales_are_pow2``.)"""
     if fp8_weight is None:
         return quantize_expert_weights(weight)
     q, s = fp8_weight
@@ -162,7 +164,7 @@ def silu_jagged_bmm_fp8(
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=True)
     qw, sw = _weight_pair(weight.permute(0, 2, 1), fp8_weight)          # rows of [E, D_out, D_in]
     return ops.grouped_gemm(seq_offsets, qa, qw, total_rows=jagged.shape[0], bias=bias,
-                            scales_pow2=True, a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
+                            scales_pow2=ops.scales_are_pow2(sa, sw), a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
 
 
 def silu_jagged_bmm_combine_fp8(
@@ -192,8 +194,8 @@ def silu_jagged_bmm_combine_fp8(
         return _ag.SiluJaggedBmmCombine.apply(offsets, jagged, weight, bias, index, reverse_index, gating_scores,
                                               gates_index, has_silu, (qw, sw), activation_checkpointing)
     qa, sa = ops.quant_rows_fp8(jagged, apply_silu=has_silu)
-    bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias, scales_pow2=True, a_scale=sa,
-                               b_scale=sw, epilogue=EPI_NONE)
+    bmm_out = ops.grouped_gemm(offsets, qa, qw, total_rows=jagged.shape[0], bias=bias,
+                               scales_pow2=ops.scales_are_pow2(sa, sw), a_scale=sa, b_scale=sw, epilogue=EPI_NONE)
     return ops.combine(bmm_out, reverse_index, gating_scores, gates_index)
 
 
@@ -226,5 +228,5 @@ def index_select_jagged_bmm(
         return _ag.IndexSelectJaggedBmmFp8.apply(offsets, index, jagged, weight, bias, (qw, sw))
     qa, sa = ops.quant_rows_fp8(jagged)
     return ops.grouped_gemm(offsets, qa, qw, total_rows=index.numel(), row_index=index,
-                            index_div=index.shape[-1], bias=bias, scales_pow2=True, a_scale=sa, b_scale=sw,
-                            epilogue=EPI_NONE)
+                            index_div=index.shape[-1], bias=bias, scales_pow2=ops.scales_are_pow2(sa, sw), a_scale=sa,
+                            b_scale=sw, epilogue=EPI_NONE)

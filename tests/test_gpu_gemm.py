@@ -307,6 +307,33 @@ def test_fp8_combine(E, K, Din, Dout, has_silu):
     assert bool((err <= 3e-2 * ref.float().abs() + 3e-2).all()), err.max()
 
 
+def test_fp8_weight_pair_of_other_origin_is_not_taken_for_powers_of_two():
+    """A caller may hand the fp8 operators its own (bytes, scales) pair.  Only scale tensors that
+    the package's quantiser returned (and nobody wrote to since) are taken for exact powers of
+    two and given to the MFMAs as block scales; any other pair has its scales divided out in the
+    epilogue, which is right for every positive scale."""
+    from fast_moe_amd.kernels import moe_fp8
+    from fast_moe_amd.kernels.hip import ops
+    L, E, K, Din, Dout = 4096, 8, 2, 256, 512
+    r = make_routing(L, E, K, seed=3)
+    x = dev(randn((L, Din), 1))
+    w = dev(weights(E, Din, Dout, 2, False, scale=Din ** -0.5))
+    offsets, index = dev(r["offsets"]), dev(r["index"])
+    qw, sw = moe_fp8.quantize_expert_weights(w)
+    assert ops.scales_are_pow2(sw)
+    other = sw * 1.5                         # a legitimate pair of other origin: same bytes, weights 1.5 times smaller
+    assert not ops.scales_are_pow2(other) and not ops.scales_are_pow2(sw.clone())
+    qa, sa = ops.quant_rows_fp8(x)
+    kw = dict(total_rows=L * K, row_index=index.reshape(-1), index_div=K, a_scale=sa)
+    want = ops.grouped_gemm(offsets, qa, qw, b_scale=other, scales_pow2=False, **kw)
+    got = moe_fp8.index_select_jagged_bmm(0, offsets, index, x, w, None, fp8=True, fp8_weight=(qw, other))
+    assert torch.equal(got, want)
+    base = moe_fp8.index_select_jagged_bmm(0, offsets, index, x, w, None, fp8=True, fp8_weight=(qw, sw))
+    assert_bf16_close(got.float() * 1.5, base.float(), rtol=1.6e-2, atol=1e-2, what="scales 1.5 times larger")
+    sw.mul_(1.0)                              # written to: no longer vouched for
+    assert not ops.scales_are_pow2(sw)
+
+
 def test_forward_only_and_dtype_errors():
     from fast_moe_amd.kernels import moe, moe_fp8
     r = make_routing(16, 4, 2)
