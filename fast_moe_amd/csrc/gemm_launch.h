@@ -12,6 +12,14 @@ typedef TileCfg<256, 256, 2, 4> TileBig;        // 8 waves, wave tile 128 x 64
 typedef TileCfg<64, 256, 1, 4> TileSmall;       // 4 waves, wave tile 64 x 64
 typedef RingCfg<256, 256, 2, 4, 0> TileRing4;   // 8 waves, wave tile 128 x 64, 4-slot ring, LDS tables
 typedef RingCfg<256, 256, 2, 4, 1> TileRing5;   // 5-slot ring, paired slices, E <= 64
+// The plain forward calls take TileRing5F.  A build with -DFMOE_RING_NARROW gives them 256 x 128 tiles
+// of 4 waves (one wave per SIMD, half the accumulator footprint per CU) instead: a measurement
+// variant, kept so that the comparison can be repeated; 16-25 % slower than the 8-wave tile.
+#ifdef FMOE_RING_NARROW
+typedef RingCfg<256, 128, 2, 2, 1> TileRing5F;
+#else
+typedef TileRing5 TileRing5F;
+#endif
 typedef RingCfg<256, 256, 2, 4, 4> TileRing5W;  // 5-slot ring, paired slices, E <= 256
 
 enum GemmKernelSel { kSelRing = 0, kSelStagedBig = 1, kSelStagedSmall = 2, kSelGeneric = 3 };
@@ -144,11 +152,11 @@ int launch_ring(const GemmParams& p, hipStream_t stream) {
     }
     if constexpr (FP8) {                   // power-of-two scales: applied by the MFMAs (row numbers fit 31 bits: pair_ok)
         if (p.scale_pow2 && pair_ok && p.E <= TileRing5::kMaxExperts)
-            return launch_ring_cfg<TileRing5, FP8, EPI, false, false, false, true>(p, stream);
+            return launch_ring_cfg<TileRing5F, FP8, EPI, false, false, false, true>(p, stream);
         if (p.scale_pow2 && pair_ok && p.E <= TileRing5W::kMaxExperts)
             return launch_ring_cfg<TileRing5W, FP8, EPI, false, false, false, true>(p, stream);
     }
-    if (pair_ok && p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5, FP8, EPI>(p, stream);
+    if (pair_ok && p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5F, FP8, EPI>(p, stream);
     if (pair_ok && p.E <= TileRing5W::kMaxExperts) return launch_ring_cfg<TileRing5W, FP8, EPI>(p, stream);
     return launch_ring_cfg<TileRing4, FP8, EPI>(p, stream);
 }

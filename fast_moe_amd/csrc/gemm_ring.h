@@ -794,17 +794,24 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                 constexpr bool DMA = decltype(dma_c)::value;
                 constexpr int ACT = decltype(act_c)::value;
                 constexpr int NM = FN * ACT;
-                static_assert(NM % L == 0 || L % NM == 0, "DMA parts must spread evenly over the MFMAs");
-                constexpr int PER = L >= NM ? L / NM : 1, EVERY = L >= NM ? 1 : NM / L;
+                // part q of the pair goes out behind MFMA ceil((q + 1) * NM / L) - 1: evenly spread
+                // whether the parts are as many as the MFMAs, a divisor or a multiple of them, or neither
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int fn = m / ACT, fm = m % ACT;
                     acc[fn][fm] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[fn], xf[fm], acc[fn][fm], 0, 0, 0);
-                    if (DMA && (m + 1) % EVERY == 0) {
-                        __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (DMA) {
+                        constexpr auto slot_of = [](int q) { return ((q + 1) * NM + L - 1) / L - 1; };
+                        bool any = false;
 #pragma unroll
-                        for (int q = 0; q < PER; ++q) issue_part(((m + 1) / EVERY - 1) * PER + q);
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int q = 0; q < L; ++q) any |= slot_of(q) == m;
+                        if (any) {
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int q = 0; q < L; ++q)
+                                if (slot_of(q) == m) issue_part(q);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     }
                 }
             };
@@ -944,8 +951,6 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                     }
                     return;
                 }
-                static_assert(NM % L == 0 || L % NM == 0, "DMA parts must spread evenly over the MFMAs");
-                constexpr int PER = L >= NM ? L / NM : 1, EVERY = L >= NM ? 1 : NM / L;
 #pragma unroll
                 for (int m = 0; m < NM; ++m) {
                     const int fn = m / HM, fm = m % HM;
@@ -962,11 +967,18 @@ __global__ __launch_bounds__(TL::NT) void grouped_gemm_ring_kernel(const GemmPar
                         acc[fn][FM0 + fm] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                             wf[fn], xh[fm], acc[fn][FM0 + fm], 0, 0, 0, 0, 0, 0);
                     }
-                    if (DMA && (m + 1) % EVERY == 0) {
-                        __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (DMA) {        // (part q behind MFMA ceil((q + 1) * NM / L) - 1, as in the bf16 loop)
+                        constexpr auto slot_of = [](int q) { return ((q + 1) * NM + L - 1) / L - 1; };
+                        bool any = false;
 #pragma unroll
-                        for (int q = 0; q < PER; ++q) issue_part(((m + 1) / EVERY - 1) * PER + q);
-                        __builtin_amdgcn_sched_barrier(0);
+                        for (int q = 0; q < L; ++q) any |= slot_of(q) == m;
+                        if (any) {
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int q = 0; q < L; ++q)
+                                if (slot_of(q) == m) issue_part(q);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     }
                 }
             };
