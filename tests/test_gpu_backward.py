@@ -459,7 +459,7 @@ def test_two_products_in_one_gemm(lens, K1, K2, N):
 
 
 def test_full_size_c3_training_step_sampled():
-    """BASELINE's bf16 configuration (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed routing with
+    """The benchmark's bf16 configuration (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed routing with
     empty experts) forward + backward through the one-call expert block.  Checked: (1) a sample
     of token gradients and the weight gradients of the smallest non-empty expert against fp32
     autograd on just those rows; (2) size-independent: gradients are linear in the incoming

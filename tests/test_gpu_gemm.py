@@ -443,7 +443,7 @@ def test_ring_kernel_is_deterministic_and_ignores_garbage_offsets():
 
 @pytest.mark.parametrize("fp8", [False, True])
 def test_full_size_c3_c4_sampled_rows(fp8):
-    """BASELINE sizes (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed, empty experts): the
+    """The benchmark sizes (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed, empty experts): the
     whole SwiGLU GEMM runs on the GPU, a sample of its rows is checked against the oracle, and
     size-independent properties hold (rows of empty experts absent, duplicate tokens give equal rows)."""
     from fast_moe_amd.kernels import moe_fp8

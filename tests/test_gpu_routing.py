@@ -75,7 +75,7 @@ def test_route_topk_nan_inf_and_equal_rows(E, dtype):
 @pytest.mark.parametrize("T,E,K,dtype", [(16384, 64, 8, torch.float32), (8192, 8, 2, torch.bfloat16),
                                          (32768, 128, 8, torch.float32)])
 def test_route_topk_full_size(T, E, K, dtype):
-    """BASELINE sizes: exact against the oracle and the permutation invariants."""
+    """The benchmark sizes: exact against the oracle and the permutation invariants."""
     got, ref = check_route(softmax_scores(T, E, 11, dtype), K)
     gi = got["gate_index"].cpu().numpy()
     assert np.array_equal(np.sort(gi), np.arange(T * K))
