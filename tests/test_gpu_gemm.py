@@ -441,6 +441,52 @@ def test_ring_kernel_is_deterministic_and_ignores_garbage_offsets():
     assert out.shape == a.shape
 
 
+@pytest.mark.parametrize("fp8", [False, True], ids=["bf16", "fp8"])
+def test_ring_kernel_repeats_bit_identically_while_another_stream_loads_the_memory_system(fp8):
+    """The ring kernel keeps its own count of the LDS-DMA in flight; a wait that is one operation
+    short would read a slot before its data has landed, and whether that shows depends on timing.
+    Both GEMMs of the benchmark sizes (SwiGLU with gather, plain), 24 launches each, while a second
+    stream copies 1 GiB back and forth: every launch must reproduce the first bit for bit."""
+    from fast_moe_amd.kernels.hip import _lib, ops
+    T, E, K, D, H = 16384, 64, 8, 2048, 1408
+    topk = skewed_topk(T, E, K, seed=11)
+    meta = o_routing.routing_metadata(topk.numpy(), E)
+    offsets, gate_index = dev(torch.from_numpy(meta["offsets"])), dev(torch.from_numpy(meta["gate_index"]))
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn(T, D, generator=g, device="cuda").to(BF16)
+    wg = (torch.randn(E, H, D, generator=g, device="cuda") * D ** -0.5).to(BF16).permute(0, 2, 1)
+    wu = (torch.randn(E, H, D, generator=g, device="cuda") * D ** -0.5).to(BF16).permute(0, 2, 1)
+    wd = (torch.randn(E, D, H, generator=g, device="cuda") * H ** -0.5).to(BF16).permute(0, 2, 1)
+    if fp8:
+        (qx, sx), (qg, sg), (qu, su), (qd, sd) = (ops.quant_rows_fp8(x), ops.quant_rows_fp8(wg.permute(0, 2, 1)),
+                                                    ops.quant_rows_fp8(wu.permute(0, 2, 1)),
+                                                    ops.quant_rows_fp8(wd.permute(0, 2, 1)))
+        gemm1 = lambda: ops.grouped_gemm(offsets, qx, qg.permute(0, 2, 1), total_rows=T * K, row_index=gate_index,
+                                         index_div=K, b2=qu.permute(0, 2, 1), epilogue=_lib.EPI_SWIGLU, a_scale=sx,
+                                         b_scale=sg, b2_scale=su, scales_pow2=True)
+    else:
+        gemm1 = lambda: ops.grouped_gemm(offsets, x, wg, total_rows=T * K, row_index=gate_index, index_div=K, b2=wu,
+                                         epilogue=_lib.EPI_SWIGLU)
+    hidden = gemm1()
+    if fp8:
+        qh, sh = ops.quant_rows_fp8(hidden)
+        gemm2 = lambda: ops.grouped_gemm(offsets, qh, qd.permute(0, 2, 1), total_rows=T * K, a_scale=sh, b_scale=sd,
+                                         scales_pow2=True)
+    else:
+        gemm2 = lambda: ops.grouped_gemm(offsets, hidden, wd, total_rows=T * K)
+    first2 = gemm2()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    a, b = torch.empty(1 << 28, dtype=torch.int32, device="cuda"), torch.empty(1 << 28, dtype=torch.int32, device="cuda")
+    for i in range(24):
+        with torch.cuda.stream(side):               # (default priority) a copy that competes for HBM and L2
+            (b if i % 2 else a).copy_(a if i % 2 else b, non_blocking=True)
+        h, o = gemm1(), gemm2()
+        assert torch.equal(h, hidden), f"gemm1, launch {i}"
+        assert torch.equal(o, first2), f"gemm2, launch {i}"
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 def test_full_size_c3_c4_sampled_rows(fp8):
     """The benchmark sizes (T=16384, E=64, top-8, D=2048, H=1408, Zipf-skewed, empty experts): the
