@@ -287,7 +287,8 @@ enum fmoe_gemm_plan {
     FMOE_PLAN_NONE = -1,          /* nothing to do (no rows)                                */
     FMOE_PLAN_RING = 0,           /* persistent LDS-ring kernel, 256 x 256 tiles            */
     FMOE_PLAN_STAGED = 1,         /* register-staged kernel, 256 x 256 tiles                */
-    FMOE_PLAN_STAGED_SHORT = 2,   /* register-staged kernel, 64 x 256 tiles (few rows per expert) */
+    FMOE_PLAN_STAGED_SHORT = 2,   /* 64 x 256 tiles (few rows per expert): the streaming kernel,
+                                     or the register-staged one where that does not apply   */
     FMOE_PLAN_ELEMENT = 3         /* element loads: any strides, any alignment              */
 };
 int fmoe_grouped_gemm_plan(const fmoe_gemm_desc* desc, int* plan);
