@@ -279,10 +279,12 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_stream_kernel(const GemmP
                         xf[fm] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
                     }
                     if constexpr (MSC) {
-                        acc[0][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[0], xf[0], acc[0][0], 0, 0, 2, (int)sc, 0, (int)sc);
-                        acc[0][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[0], xf[1], acc[0][1], 0, 0, 2, (int)sc, 1, (int)sc);
-                        acc[1][0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[1], xf[0], acc[1][0], 0, 0, 3, (int)sc, 0, (int)sc);
-                        acc[1][1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[1], xf[1], acc[1][1], 0, 0, 3, (int)sc, 1, (int)sc);
+                        // (the accumulator tied to the destination, as in the ring kernel: through the
+                        // builtin it is a separate early-clobber operand and the kernel spills)
+                        mfma_e4m3_scaled<2, 0>(wf[0], xf[0], acc[0][0], sc, sc);
+                        mfma_e4m3_scaled<2, 1>(wf[0], xf[1], acc[0][1], sc, sc);
+                        mfma_e4m3_scaled<3, 0>(wf[1], xf[0], acc[1][0], sc, sc);
+                        mfma_e4m3_scaled<3, 1>(wf[1], xf[1], acc[1][1], sc, sc);
                     } else {
 #pragma unroll
                         for (int fn = 0; fn < FN; ++fn)
@@ -306,6 +308,7 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_stream_kernel(const GemmP
             fetch_rows(nxt, raw, sraw);
         }
         multiply((KT - 1) & 1);
+        if constexpr (MSC) mfma_results_guard();    // the last MFMAs' results are read by VALU code from here on
         __syncthreads();                    // every wave is done with the stages before the next tile fills stage 0
 
         // the next tile's first K-slice (and its scales) go out ahead of this tile's stores
