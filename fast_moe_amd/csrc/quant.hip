@@ -84,7 +84,9 @@ __device__ __forceinline__ u32x2 encode8(const u32x4& v, float s, bool special) 
 }
 
 // ---- fast path: bf16, contiguous columns, cols % 8 == 0, <= CH*512 columns
-template <int CH, bool SILU>
+// W16: a lane takes pairs of neighbouring 16-byte chunks (32 contiguous input bytes), so that its
+// eight-byte results pair up into one 16-byte store (rows of a whole number of such pairs)
+template <int CH, bool SILU, bool W16 = false>
 __global__ __launch_bounds__(256) void quant_rows_bf16_wave(
     const uint16_t* __restrict__ a, int64_t total_rows, int64_t rows, int cols, int64_t a_sb,
     int64_t a_sr, uint8_t* __restrict__ q, int64_t q_sb, int64_t q_sr, float* __restrict__ scale,
@@ -97,10 +99,13 @@ __global__ __launch_bounds__(256) void quant_rows_bf16_wave(
     uint8_t* dst = q + b * q_sb + r * q_sr;
     const int chunks = cols >> 3;
 
+    static_assert(!W16 || CH % 2 == 0, "pairs of chunks");
+    // chunk held in v[i]
+    auto chunk_of = [&](int i) { return W16 ? 2 * (lane + kWave * (i / 2)) + (i & 1) : lane + kWave * i; };
     u32x4 v[CH];
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
-        const int c = lane + kWave * i;
+        const int c = chunk_of(i);
         v[i] = c < chunks ? *reinterpret_cast<const u32x4*>(src + (int64_t)c * 8) : u32x4{0, 0, 0, 0};
     }
     float m = 0.0f;
@@ -124,12 +129,22 @@ __global__ __launch_bounds__(256) void quant_rows_bf16_wave(
     const float s = scale_from_amax<true>(m);   // every element is a bf16 value
     if (lane == 0) scale[row] = store_reciprocal ? 1.0f / s : s;
     const bool special = !(m <= 3.4028234664e38f);   // NaN or inf in the row
+    if constexpr (W16) {
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-        const int c = lane + kWave * i;
-        if (c >= chunks) continue;
-        const u32x2 o = encode8(v[i], s, special);
-        *reinterpret_cast<u32x2*>(dst + (int64_t)c * 8) = o;
+        for (int i = 0; i < CH; i += 2) {
+            const int c = chunk_of(i);
+            if (c >= chunks) continue;
+            const u32x2 lo = encode8(v[i], s, special), hi = encode8(v[i + 1], s, special);
+            *reinterpret_cast<u32x4*>(dst + (int64_t)c * 8) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            const int c = lane + kWave * i;
+            if (c >= chunks) continue;
+            const u32x2 o = encode8(v[i], s, special);
+            *reinterpret_cast<u32x2*>(dst + (int64_t)c * 8) = o;
+        }
     }
 }
 
@@ -243,11 +258,23 @@ __global__ __launch_bounds__(256) void quant_rows_generic_lane(
         dst[c * q_sc] = (uint8_t)e4m3fn_encode(fetch<T, SILU>(src + c * a_sc) * s);
 }
 
+// rows that are whole pairs of chunks, stored 16 bytes at a time
+inline bool wide_stores(bool silu, int64_t cols, const uint8_t* q, int64_t q_sb, int64_t q_sr) {
+    return !silu && cols % 16 == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0 && q_sb % 16 == 0 && q_sr % 16 == 0;
+}
+
 template <int CH>
 void launch_fast(bool silu, const uint16_t* a, int64_t total, int64_t rows, int cols, int64_t a_sb,
                  int64_t a_sr, uint8_t* q, int64_t q_sb, int64_t q_sr, float* scale, int recip,
                  hipStream_t stream) {
     const unsigned blocks = (unsigned)((total + 3) / 4);
+    if constexpr (CH % 2 == 0) {
+        if (wide_stores(silu, cols, q, q_sb, q_sr)) {
+            quant_rows_bf16_wave<CH, false, true><<<blocks, 256, 0, stream>>>(a, total, rows, cols, a_sb, a_sr, q,
+                                                                              q_sb, q_sr, scale, recip);
+            return;
+        }
+    }
     if (silu)
         quant_rows_bf16_wave<CH, true><<<blocks, 256, 0, stream>>>(a, total, rows, cols, a_sb, a_sr, q,
                                                                    q_sb, q_sr, scale, recip);
@@ -298,7 +325,8 @@ extern "C" int fmoe_quant_rows_e4m3(const void* a, int a_dtype, int64_t batch, i
                       cols <= 16 * 512 && aligned16(a) && (a_sb % 8) == 0 && (a_sr % 8) == 0 &&
                       (reinterpret_cast<uintptr_t>(q) & 7u) == 0 && (q_sb % 8) == 0 && (q_sr % 8) == 0;
     if (fast) {
-        const int ch = (int)((cols / 8 + kWave - 1) / kWave);
+        int ch = (int)((cols / 8 + kWave - 1) / kWave);
+        if (wide_stores(apply_silu != 0, cols, q, q_sb, q_sr)) ch = 2 * (int)((cols / 16 + kWave - 1) / kWave);
 #define FMOE_FAST(CH)                                                                              \
     launch_fast<CH>(apply_silu != 0, (const uint16_t*)a, total, rows, (int)cols, a_sb, a_sr, q, q_sb, \
                     q_sr, scale, store_reciprocal, stream)
