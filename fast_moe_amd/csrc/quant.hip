@@ -259,8 +259,8 @@ __global__ __launch_bounds__(256) void quant_rows_generic_lane(
 }
 
 // rows that are whole pairs of chunks, stored 16 bytes at a time
-inline bool wide_stores(bool silu, int64_t cols, const uint8_t* q, int64_t q_sb, int64_t q_sr) {
-    return !silu && cols % 16 == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0 && q_sb % 16 == 0 && q_sr % 16 == 0;
+inline bool wide_stores(int64_t cols, const uint8_t* q, int64_t q_sb, int64_t q_sr) {
+    return cols % 16 == 0 && (reinterpret_cast<uintptr_t>(q) & 15u) == 0 && q_sb % 16 == 0 && q_sr % 16 == 0;
 }
 
 template <int CH>
@@ -269,9 +269,13 @@ void launch_fast(bool silu, const uint16_t* a, int64_t total, int64_t rows, int 
                  hipStream_t stream) {
     const unsigned blocks = (unsigned)((total + 3) / 4);
     if constexpr (CH % 2 == 0) {
-        if (wide_stores(silu, cols, q, q_sb, q_sr)) {
-            quant_rows_bf16_wave<CH, false, true><<<blocks, 256, 0, stream>>>(a, total, rows, cols, a_sb, a_sr, q,
-                                                                              q_sb, q_sr, scale, recip);
+        if (wide_stores(cols, q, q_sb, q_sr)) {
+            if (silu)
+                quant_rows_bf16_wave<CH, true, true><<<blocks, 256, 0, stream>>>(a, total, rows, cols, a_sb, a_sr, q,
+                                                                                 q_sb, q_sr, scale, recip);
+            else
+                quant_rows_bf16_wave<CH, false, true><<<blocks, 256, 0, stream>>>(a, total, rows, cols, a_sb, a_sr, q,
+                                                                                  q_sb, q_sr, scale, recip);
             return;
         }
     }
@@ -326,7 +330,7 @@ extern "C" int fmoe_quant_rows_e4m3(const void* a, int a_dtype, int64_t batch, i
                       (reinterpret_cast<uintptr_t>(q) & 7u) == 0 && (q_sb % 8) == 0 && (q_sr % 8) == 0;
     if (fast) {
         int ch = (int)((cols / 8 + kWave - 1) / kWave);
-        if (wide_stores(apply_silu != 0, cols, q, q_sb, q_sr)) ch = 2 * (int)((cols / 16 + kWave - 1) / kWave);
+        if (wide_stores(cols, q, q_sb, q_sr)) ch = 2 * (int)((cols / 16 + kWave - 1) / kWave);
 #define FMOE_FAST(CH)                                                                              \
     launch_fast<CH>(apply_silu != 0, (const uint16_t*)a, total, rows, (int)cols, a_sb, a_sr, q, q_sb, \
                     q_sr, scale, store_reciprocal, stream)
