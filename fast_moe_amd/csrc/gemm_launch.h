@@ -20,6 +20,7 @@ typedef RingCfg<256, 128, 2, 2, 1> TileRing5F;
 #else
 typedef TileRing5 TileRing5F;
 #endif
+typedef RingCfg<256, 256, 2, 4, 2> TileRing5M;  // 5-slot ring, paired slices, E <= 128 (the plain forward calls)
 typedef RingCfg<256, 256, 2, 4, 4> TileRing5W;  // 5-slot ring, paired slices, E <= 256
 
 enum GemmKernelSel { kSelRing = 0, kSelStagedBig = 1, kSelStagedSmall = 2, kSelGeneric = 3 };
@@ -153,10 +154,13 @@ int launch_ring(const GemmParams& p, hipStream_t stream) {
     if constexpr (FP8) {                   // power-of-two scales: applied by the MFMAs (row numbers fit 31 bits: pair_ok)
         if (p.scale_pow2 && pair_ok && p.E <= TileRing5::kMaxExperts)
             return launch_ring_cfg<TileRing5F, FP8, EPI, false, false, false, true>(p, stream);
+        if (p.scale_pow2 && pair_ok && p.E <= TileRing5M::kMaxExperts)
+            return launch_ring_cfg<TileRing5M, FP8, EPI, false, false, false, true>(p, stream);
         if (p.scale_pow2 && pair_ok && p.E <= TileRing5W::kMaxExperts)
             return launch_ring_cfg<TileRing5W, FP8, EPI, false, false, false, true>(p, stream);
     }
     if (pair_ok && p.E <= TileRing5::kMaxExperts) return launch_ring_cfg<TileRing5F, FP8, EPI>(p, stream);
+    if (pair_ok && p.E <= TileRing5M::kMaxExperts) return launch_ring_cfg<TileRing5M, FP8, EPI>(p, stream);
     if (pair_ok && p.E <= TileRing5W::kMaxExperts) return launch_ring_cfg<TileRing5W, FP8, EPI>(p, stream);
     return launch_ring_cfg<TileRing4, FP8, EPI>(p, stream);
 }
